@@ -45,3 +45,6 @@ class ForwardBatch:
     tile_seq: Optional[torch.Tensor] = None   # [n_tiles] int32 seq index
     tile_q0: Optional[torch.Tensor] = None    # [n_tiles] int32 local row start
     prefill_token_count: int = 0              # flat rows belonging to prefills
+    # models with per-sequence recurrent state / per-token sequence lookups
+    state_slots: Optional[torch.Tensor] = None  # [S] int32 state slot per seq
+    token_seq: Optional[torch.Tensor] = None    # [T] int32 seq index per row

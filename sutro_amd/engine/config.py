@@ -65,24 +65,23 @@ class EngineConfig:
         if self.max_model_len > self.spec.max_context:
             self.max_model_len = self.spec.max_context
 
-    def derive_num_kv_blocks(self, free_bytes: int) -> int:
-        """KV blocks that fit in `free_bytes` (both K and V, all layers)."""
+    def derive_num_kv_blocks(self, free_bytes: int, layer_shapes=None) -> int:
+        """KV blocks that fit in `free_bytes` (both K and V, all layers).
+        `layer_shapes`: per layer (kv_heads, key_dim, value_dim) or None for a
+        layer without keys; default = the spec's uniform layout."""
         spec = self.spec
-        kvh = spec.num_kv_heads // self.tp_size if spec.num_kv_heads >= self.tp_size else 1
         if self.kv_dtype == "fp8_e4m3":
             elem = 1
         elif self.dtype in (torch.bfloat16, torch.float16):
             elem = 2
         else:
             elem = 4
-        bytes_per_block = (
-            2  # K and V
-            * spec.num_layers
-            * kvh
-            * self.kv_block_size
-            * spec.head_dim
-            * elem
-        )
+        if layer_shapes is None:
+            kvh = spec.num_kv_heads // self.tp_size if spec.num_kv_heads >= self.tp_size else 1
+            layer_shapes = [(kvh, spec.head_dim, spec.head_dim)] * spec.num_layers
+        per_token = sum(s[0] * (s[1] + s[2]) for s in layer_shapes
+                        if s is not None)
+        bytes_per_block = max(1, per_token * self.kv_block_size * elem)
         return max(16, int(free_bytes // bytes_per_block))
 
     def kv_torch_dtype(self) -> torch.dtype:

@@ -21,12 +21,11 @@ from typing import Dict, List, Optional
 import numpy as np
 import torch
 
-from ..models.qwen3 import Qwen3Model
-from ..models.registry import ModelSpec
+from ..models.registry import ModelSpec, build_model
 from .batch import ForwardBatch, ScheduledBatch
 from .config import EngineConfig
 from .guided import GuidedFSM
-from .kv_cache import PagedKVCache
+from .kv_cache import PagedKVCache, RecurrentStateCache
 from .request import FinishReason, Request, SamplingParams
 from .sampler import Sampler
 from .scheduler import Scheduler
@@ -82,22 +81,37 @@ class LLMEngine:
                    else TPContext())
         if model is None:
             with torch.device(cfg.device):
-                model = Qwen3Model(self.spec, cfg.dtype, cfg.max_model_len,
-                                   self.tp, moe_ep=cfg.moe_ep)
-            if cfg.weights_path:
+                model = build_model(self.spec, cfg.dtype, cfg.max_model_len,
+                                    self.tp, moe_ep=cfg.moe_ep)
+            weights = cfg.weights_path or getattr(self.spec, "checkpoint_dir",
+                                                  None)
+            if weights:
                 from ..models.loader import load_weights
 
-                load_weights(model, cfg.weights_path)
+                load_weights(model, weights)
             else:
                 model.init_random_weights(cfg.seed)
         self.model = model.to(cfg.device).eval()
+
+        # cache layout: uniform (heads, head_dim) for the Qwen3 family; models
+        # with their own per-layer key/value sizes or recurrent state say so
+        if hasattr(self.model, "cache_layout"):
+            kv_shapes, state_shapes = self.model.cache_layout()
+        else:
+            kvh = self.spec.num_kv_heads
+            if cfg.tp_size > 1:
+                kvh = max(1, kvh // cfg.tp_size)
+            kv_shapes = [(kvh, self.spec.head_dim, self.spec.head_dim)
+                         ] * self.spec.num_layers
+            state_shapes = None
 
         num_blocks = cfg.num_kv_blocks
         if num_blocks is None:
             if cfg.device.startswith("cuda"):
                 free, total = torch.cuda.mem_get_info()
                 headroom = int((1.0 - cfg.gpu_memory_utilization) * total)
-                num_blocks = cfg.derive_num_kv_blocks(max(0, free - headroom))
+                num_blocks = cfg.derive_num_kv_blocks(max(0, free - headroom),
+                                                      kv_shapes)
                 # cap the block-table width the scheduler can ever need
                 max_blocks_useful = (
                     (cfg.max_model_len + cfg.kv_block_size - 1) // cfg.kv_block_size
@@ -105,17 +119,21 @@ class LLMEngine:
                 num_blocks = min(num_blocks, max_blocks_useful)
             else:
                 num_blocks = 1024
-        kvh = self.spec.num_kv_heads
-        if cfg.tp_size > 1:
-            kvh = max(1, kvh // cfg.tp_size)
+        state = None
+        if state_shapes is not None and any(s is not None for s in state_shapes):
+            state = RecurrentStateCache(cfg.max_num_seqs, state_shapes,
+                                        cfg.device)
+        first = next((s for s in kv_shapes if s is not None), (1, 1, 1))
         self.kv = PagedKVCache(
             num_layers=self.spec.num_layers,
             num_blocks=num_blocks,
-            num_kv_heads=kvh,
+            num_kv_heads=first[0],
             block_size=cfg.kv_block_size,
-            head_dim=self.spec.head_dim,
+            head_dim=first[1],
             dtype=cfg.kv_torch_dtype(),
             device=cfg.device,
+            layer_shapes=kv_shapes,
+            state=state,
         )
         # block 0 is reserved scratch: hipGraph padding rows read/write it
         self.scratch_block = self.kv.allocator.allocate(1)[0]
@@ -151,7 +169,7 @@ class LLMEngine:
 
         self.prefill_graph = None
         if (cfg.graph_prefill and cfg.device.startswith("cuda")
-                and not cfg.enforce_eager):
+                and not cfg.enforce_eager and self.kv.state is None):
             from .prefill_graph import PrefillGraphRunner
 
             try:
@@ -285,7 +303,17 @@ class LLMEngine:
         prefill_token_count = int(qlocs[sb.num_prefills])
 
         dev = self.device
+        state_slots = token_seq = None
+        if self.kv.state is not None:
+            slots_of = self.kv.state.slots
+            state_slots = torch.tensor([slots_of[r.req_id] for r in sb.reqs],
+                                       dtype=torch.int32, device=dev)
+            token_seq = torch.from_numpy(np.repeat(
+                np.arange(S, dtype=np.int32),
+                np.asarray(sb.num_new_tokens, dtype=np.int64))).to(dev)
         return ForwardBatch(
+            state_slots=state_slots,
+            token_seq=token_seq,
             input_ids=torch.from_numpy(input_ids).to(dev),
             positions=torch.from_numpy(positions).to(dev),
             slot_mapping=torch.from_numpy(slots).to(dev),
@@ -457,6 +485,80 @@ class LLMEngine:
         self.total_prompt_tokens += stats.prefill_tokens
         self.total_output_tokens += stats.output_tokens
         return stats
+
+    # ---- replay of a recorded schedule (no sampling) ----
+
+    def new_replay_request(self) -> Request:
+        """A request whose tokens are supplied step by step by `replay_step`
+        (it is admitted by the scheduler at its first step)."""
+        req = Request(req_id=self._next_req_id, prompt_token_ids=[],
+                      sampling=SamplingParams(max_tokens=1))
+        self._next_req_id += 1
+        return req
+
+    @torch.no_grad()
+    def replay_step(self, entries) -> Optional[torch.Tensor]:
+        """Run one step of a recorded schedule: `entries` is a list of
+        (request, next tokens, positions among them whose logits are wanted).
+        All entries form one scheduler batch and run exactly as in `step()`
+        (prefill chunks eager, decode rows through the decode hipGraph when
+        one is captured), but nothing is sampled: the next tokens are given.
+        Returns fp32 logits [wanted, vocab] in entry order, or None."""
+        want_of: Dict[int, List[int]] = {}
+        for req, toks, want in entries:
+            req.prompt_token_ids.extend(int(t) for t in toks)
+            want_of[id(req)] = list(want)
+        sb = self.scheduler.schedule_explicit(
+            [(req, len(toks)) for req, toks, _ in entries])
+        subs: List[ScheduledBatch] = []
+        if self.graph_runner is not None and sb.num_decodes > 0 \
+                and sb.num_prefills > 0:
+            subs.append(ScheduledBatch(
+                reqs=sb.reqs[: sb.num_prefills],
+                num_new_tokens=sb.num_new_tokens[: sb.num_prefills],
+                num_prefills=sb.num_prefills))
+            subs.append(ScheduledBatch(
+                reqs=sb.reqs[sb.num_prefills:],
+                num_new_tokens=[1] * sb.num_decodes, num_prefills=0))
+        elif sb.reqs:
+            subs.append(sb)
+        got: Dict[int, torch.Tensor] = {}
+        for sub in subs:
+            rows: List[int] = []
+            owners: List[Request] = []
+            cum = 0
+            for req, c in zip(sub.reqs, sub.num_new_tokens):
+                for w in want_of[id(req)]:
+                    rows.append(cum + w)
+                    owners.append(req)
+                cum += c
+            if self.graph_runner is not None and self.graph_runner.can_run(sub):
+                logits = self.graph_runner.run(sub)
+                if rows:
+                    logits = logits[torch.tensor(rows, dtype=torch.long,
+                                                 device=logits.device)]
+            else:
+                fb = self._build_forward_batch(sub)
+                hidden = self.model(fb, self.kv)
+                logits = None
+                if rows:
+                    idx = torch.tensor(rows, dtype=torch.long,
+                                       device=hidden.device)
+                    logits = self.model.compute_logits(hidden[idx])
+            self._advance_computed(sub)
+            if rows:
+                logits = logits.float()
+                k = 0
+                for req in sub.reqs:
+                    n = len(want_of[id(req)])
+                    if n:
+                        got[id(req)] = logits[k:k + n]
+                        k += n
+        parts = [got[id(req)] for req, _, want in entries if len(want)]
+        return torch.cat(parts, dim=0) if parts else None
+
+    def finish_replay_request(self, req: Request) -> None:
+        self.scheduler.finish(req, FinishReason.STOP)
 
     def _advance_computed(self, sb: ScheduledBatch) -> None:
         for req, c in zip(sb.reqs, sb.num_new_tokens):

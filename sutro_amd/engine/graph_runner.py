@@ -49,6 +49,11 @@ class DecodeGraphRunner:
         self.d_sl = torch.ones(B, dtype=torch.int32, device=dev)
         self.d_qlocs = torch.arange(B + 1, dtype=torch.int32, device=dev)
         self.d_tiles = torch.empty(0, dtype=torch.int32, device=dev)
+        # recurrent-state models: state slot per row (padding rows use the
+        # state cache's scratch slot and start from position 0 = zero state)
+        self.has_state = engine.kv.state is not None
+        self.d_state = torch.zeros(B, dtype=torch.int32, device=dev)
+        self.h_state = torch.zeros(B, dtype=torch.int32, pin_memory=True)
         # pinned host staging
         self.h_ids = torch.zeros(B, dtype=torch.long, pin_memory=True)
         self.h_pos = torch.zeros(B, dtype=torch.long, pin_memory=True)
@@ -88,6 +93,8 @@ class DecodeGraphRunner:
             tile_seq=self.d_tiles,
             tile_q0=self.d_tiles,
             prefill_token_count=0,
+            state_slots=self.d_state[:n] if self.has_state else None,
+            token_seq=self.d_qlocs[:n] if self.has_state else None,
         )
 
     @torch.no_grad()
@@ -132,6 +139,9 @@ class DecodeGraphRunner:
         self.d_slots[:bucket].copy_(self.h_slots[:bucket], non_blocking=True)
         self.d_bt[:bucket].copy_(self.h_bt[:bucket], non_blocking=True)
         self.d_sl[:bucket].copy_(self.h_sl[:bucket], non_blocking=True)
+        if self.has_state:
+            self.d_state[:bucket].copy_(self.h_state[:bucket],
+                                        non_blocking=True)
         if ids_override is not None:
             self.d_ids[:n].copy_(ids_override, non_blocking=True)
         if self._h2d_done is not None:
@@ -184,6 +194,12 @@ class DecodeGraphRunner:
         rows = self._arange[:n]
         slots[:n] = bt[rows, p // bs].astype(np.int64) * bs + p % bs
 
+        if self.has_state:
+            st = self.h_state.numpy()
+            slots_of = kv.state.slots
+            st[:n] = np.fromiter((slots_of[r.req_id] for r in sb.reqs),
+                                 np.int32, n)
+            st[n:bucket] = kv.state.scratch_slot
         if n < bucket:  # padding rows target the reserved scratch block
             ids[n:bucket] = 0
             pos[n:bucket] = 0

@@ -1,4 +1,5 @@
-"""Paged KV cache: block allocator + per-layer page tensors.
+"""Paged KV cache: block allocator + per-layer page tensors, plus the
+fixed-size recurrent state of layers that carry one (slot per sequence).
 
 Layout (per layer, K and V separate):
     cache[num_blocks, num_kv_heads, block_size, head_dim]
@@ -10,7 +11,7 @@ new token's K/V row with a single dwordx4-per-lane store.
 
 from __future__ import annotations
 
-from typing import Dict, List
+from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
@@ -35,6 +36,57 @@ class BlockAllocator:
         self._free.extend(reversed(blocks))
 
 
+class RecurrentStateCache:
+    """Per-sequence fixed-size state of recurrent mixers, one slot a sequence.
+
+    For every layer that carries state (`shapes[i]` = (channels, taps, heads,
+    dk, dv), else None):
+        conv[i]  [slots, taps-1, channels] fp32 — the last taps-1 inputs of the
+                 layer's short filters, oldest first;
+        ssm[i]   [slots, heads, dk, dv] fp32 — the delta-rule memory.
+    A slot is not cleared when it is handed out again: the kernels start from
+    zero whenever a sequence's first token (position 0) is in the batch.
+    Slot 0 is reserved as scratch for padded graph rows."""
+
+    def __init__(self, num_slots: int,
+                 shapes: Sequence[Optional[Tuple[int, int, int, int, int]]],
+                 device: str) -> None:
+        self.num_slots = num_slots + 1
+        self.conv: List[Optional[torch.Tensor]] = []
+        self.ssm: List[Optional[torch.Tensor]] = []
+        for sh in shapes:
+            if sh is None:
+                self.conv.append(None)
+                self.ssm.append(None)
+                continue
+            ch, taps, heads, dk, dv = sh
+            self.conv.append(torch.zeros(self.num_slots, max(1, taps - 1), ch,
+                                         dtype=torch.float32, device=device))
+            self.ssm.append(torch.zeros(self.num_slots, heads, dk, dv,
+                                        dtype=torch.float32, device=device))
+        self.scratch_slot = 0
+        self._free: List[int] = list(range(self.num_slots - 1, 0, -1))
+        self.slots: Dict[int, int] = {}
+
+    @property
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def acquire(self, req_id: int) -> int:
+        slot = self.slots.get(req_id)
+        if slot is None:
+            if not self._free:
+                raise MemoryError("recurrent state slots exhausted")
+            slot = self._free.pop()
+            self.slots[req_id] = slot
+        return slot
+
+    def release(self, req_id: int) -> None:
+        slot = self.slots.pop(req_id, None)
+        if slot is not None:
+            self._free.append(slot)
+
+
 class PagedKVCache:
     def __init__(
         self,
@@ -45,20 +97,35 @@ class PagedKVCache:
         head_dim: int,
         dtype: torch.dtype,
         device: str,
+        layer_shapes: Optional[Sequence[Optional[Tuple[int, int, int]]]] = None,
+        state: Optional[RecurrentStateCache] = None,
     ) -> None:
+        """`layer_shapes`, when given, sizes every layer by itself:
+        (kv_heads, key_dim, value_dim), or None for a layer without keys
+        (its k_cache/v_cache entries are None). `state` ties recurrent-state
+        slots to the life of a sequence's pages."""
         self.num_layers = num_layers
         self.num_blocks = num_blocks
         self.num_kv_heads = num_kv_heads
         self.block_size = block_size
         self.head_dim = head_dim
-        shape = (num_blocks, num_kv_heads, block_size, head_dim)
-        self.k_cache = [
-            torch.zeros(shape, dtype=dtype, device=device) for _ in range(num_layers)
-        ]
-        self.v_cache = [
-            torch.zeros(shape, dtype=dtype, device=device) for _ in range(num_layers)
-        ]
+        if layer_shapes is None:
+            layer_shapes = [(num_kv_heads, head_dim, head_dim)] * num_layers
+        self.layer_shapes = list(layer_shapes)
+        self.k_cache: List[Optional[torch.Tensor]] = []
+        self.v_cache: List[Optional[torch.Tensor]] = []
+        for sh in self.layer_shapes:
+            if sh is None:
+                self.k_cache.append(None)
+                self.v_cache.append(None)
+                continue
+            kvh, kd, vd = sh
+            self.k_cache.append(torch.zeros((num_blocks, kvh, block_size, kd),
+                                            dtype=dtype, device=device))
+            self.v_cache.append(torch.zeros((num_blocks, kvh, block_size, vd),
+                                            dtype=dtype, device=device))
         self.allocator = BlockAllocator(num_blocks)
+        self.state = state
         # per-sequence block tables (python side; tensorized per step)
         self.block_tables: Dict[int, List[int]] = {}
 
@@ -67,10 +134,15 @@ class PagedKVCache:
 
     def can_grow(self, req_id: int, new_len: int) -> bool:
         have = len(self.block_tables.get(req_id, []))
+        if (self.state is not None and req_id not in self.state.slots
+                and self.state.num_free == 0):
+            return False
         return self.blocks_needed(new_len) - have <= self.allocator.num_free
 
     def grow(self, req_id: int, new_len: int) -> None:
         """Ensure the sequence has pages covering new_len tokens."""
+        if self.state is not None:
+            self.state.acquire(req_id)
         table = self.block_tables.setdefault(req_id, [])
         need = self.blocks_needed(new_len) - len(table)
         if need > 0:
@@ -80,6 +152,8 @@ class PagedKVCache:
         table = self.block_tables.pop(req_id, None)
         if table:
             self.allocator.free(table)
+        if self.state is not None:
+            self.state.release(req_id)
 
     def slot(self, req_id: int, pos: int) -> int:
         """Flat slot index for token position `pos` of a sequence."""

@@ -85,6 +85,38 @@ class Scheduler:
                 if not self._preempt_one(req, scheduled):
                     return False
 
+    def schedule_explicit(self, plan) -> ScheduledBatch:
+        """Build the batch a recorded schedule dictates instead of choosing
+        one: `plan` is a list of (request, number of new tokens). Admission,
+        page growth and state slots go through the same cache manager as
+        `schedule()`; nothing is preempted (a plan that does not fit raises
+        MemoryError). Rows of one token that continue a sequence are decode
+        rows, everything else is a prefill chunk; prefills come first."""
+        prefill: List[tuple] = []
+        decode: List[Request] = []
+        for req, n in plan:
+            if n <= 0:
+                continue
+            if req not in self.running:
+                if len(self.running) >= self.cfg.max_num_seqs:
+                    raise MemoryError("no free sequence slot for the plan")
+                for q in (self.waiting_p0, self.waiting_p1):
+                    try:
+                        q.remove(req)
+                    except ValueError:
+                        pass
+                self.priorities.setdefault(req.req_id, 0)
+                self.running.append(req)
+            self.kv.grow(req.req_id, req.num_computed_tokens + n)
+            if n == 1 and req.num_computed_tokens > 0:
+                decode.append(req)
+            else:
+                prefill.append((req, n))
+        return ScheduledBatch(
+            reqs=[r for r, _ in prefill] + decode,
+            num_new_tokens=[n for _, n in prefill] + [1] * len(decode),
+            num_prefills=len(prefill))
+
     def schedule(self) -> ScheduledBatch:
         budget = self.cfg.max_tokens_per_step
         prefill_reqs: List[Request] = []

@@ -1,0 +1,198 @@
+"""Specs for layer-list ("hybrid") decoders: every layer names its own token
+mixer and feed-forward, so attention layers, recurrent layers and layers that
+run both side by side can be ordered freely.
+
+A spec is built from a checkpoint's ``config.json`` (see :func:`vodinex_spec`)
+or directly in code (tests, benchmarks). Nothing here fixes a size: widths,
+head counts, mask sizes, filter lengths and the order of layers all come from
+the config.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional, Tuple, Union
+
+
+@dataclass(frozen=True)
+class AttnMixerSpec:
+    """Softmax attention with grouped key/value heads over a local mask.
+
+    ``chunk``: a query at position i sees keys j <= i with
+    ``j // chunk == i // chunk`` (0 = no chunking). ``window``: a query sees
+    at most the last ``window`` keys (0 = unlimited). Both may be combined.
+    ``rot_dims``: how many leading dimensions of each head are rotated
+    (rotate-half pairing inside that prefix); 0 = no rotation."""
+
+    heads: int
+    kv_heads: int
+    dim: int                 # per-head query/key size
+    vdim: int                # per-head value size
+    scale: float
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    chunk: int = 0
+    window: int = 0
+    qk_norm: bool = True
+    bias: bool = True        # q/k/v/o projections carry biases
+    out_gate: bool = True    # one sigmoid gate per head on the attention output
+
+
+@dataclass(frozen=True)
+class DeltaMixerSpec:
+    """Gated delta rule with one decay per head and key channel, fed through
+    short causal depthwise filters. ``decay_rank``/``gate_rank`` are the inner
+    sizes of the two low-rank projections (read from the checkpoint)."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int                # filter taps (the last tap is the current token)
+    decay_rank: int = 0
+    gate_rank: int = 0
+
+
+@dataclass(frozen=True)
+class ParallelMixerSpec:
+    """An attention mixer and a delta-rule mixer reading the same input; the
+    result is ``left_scale * left + right_scale * right``."""
+
+    left: AttnMixerSpec
+    right: DeltaMixerSpec
+    left_scale: float
+    right_scale: float
+
+
+MixerSpec = Union[AttnMixerSpec, DeltaMixerSpec, ParallelMixerSpec]
+
+
+@dataclass(frozen=True)
+class HybridLayerSpec:
+    kind: str                # the config's layer type
+    mixer: MixerSpec
+    ff: int = 0              # 0 = the layer has no feed-forward sublayer
+    ff_kind: str = "dense"
+
+
+@dataclass(frozen=True)
+class HybridSpec:
+    """Engine-facing spec of a layer-list decoder (the counterpart of
+    ``registry.ModelSpec`` for the uniform Qwen3 family)."""
+
+    name: str
+    arch: str
+    hidden_size: int
+    vocab_size: int
+    layers: Tuple[HybridLayerSpec, ...]
+    norm_eps: float = 1e-6
+    residual_mult: float = 1.0
+    max_context: int = 32768
+    checkpoint_dir: Optional[str] = None
+    # behavior flags shared with ModelSpec
+    reasoning: bool = False
+    embedding: bool = False
+    tie_embeddings: bool = False
+    recommended_tp: int = 1
+    num_experts: int = 0
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    def param_count(self) -> int:
+        h = self.hidden_size
+        n = 2 * self.vocab_size * h
+
+        def delta(m: DeltaMixerSpec) -> int:
+            qk = 2 * m.kv_heads * m.dim
+            v = m.heads * m.vdim
+            return (h * (qk + v + m.heads + m.decay_rank + m.gate_rank)
+                    + m.decay_rank * m.heads * m.dim + m.gate_rank * v
+                    + v * h + (qk + v) * m.conv)
+
+        def attn(m: AttnMixerSpec) -> int:
+            return h * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)
+                        + m.heads) + m.heads * m.vdim * h
+
+        for layer in self.layers:
+            m = layer.mixer
+            if isinstance(m, ParallelMixerSpec):
+                n += attn(m.left) + delta(m.right)
+            elif isinstance(m, AttnMixerSpec):
+                n += attn(m)
+            else:
+                n += delta(m)
+            n += h * h                      # residual gate of the mixer
+            if layer.ff:
+                n += 3 * h * layer.ff + h * h
+        return n
+
+    def active_param_count(self) -> int:
+        return self.param_count()
+
+
+def _delta_from_config(m: dict, ranks: Tuple[int, int]) -> DeltaMixerSpec:
+    return DeltaMixerSpec(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]),
+                          dim=int(m["dim"]), vdim=int(m["vdim"]),
+                          conv=int(m["conv"]), decay_rank=ranks[0],
+                          gate_rank=ranks[1])
+
+
+def _attn_from_config(m: dict) -> AttnMixerSpec:
+    rot = m.get("rot") or {}
+    mask = m.get("mask") or {}
+    return AttnMixerSpec(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]),
+                         dim=int(m["dim"]), vdim=int(m["vdim"]),
+                         scale=float(m["scale"]),
+                         rot_dims=int(rot.get("dims", 0)),
+                         rot_base=float(rot.get("base", 10000.0)),
+                         chunk=int(mask.get("size", 0)))
+
+
+def vodinex_spec(config: dict, name: str = "vodinex",
+                 checkpoint_dir: Optional[str] = None,
+                 tensor_shapes: Optional[dict] = None) -> HybridSpec:
+    """Build the spec of a Vodinex checkpoint from its ``config.json``.
+
+    The inner sizes of the low-rank decay and gate projections are not in the
+    config; they are the row counts of ``<mixer>.a1`` / ``<mixer>.g1`` and are
+    taken from ``tensor_shapes`` (tensor name -> shape). Callers that build a
+    model in code pass them in the layer's mixer dict as ``decay_rank`` /
+    ``gate_rank`` instead."""
+    shapes = tensor_shapes or {}
+
+    def ranks(prefix: str, m: dict) -> Tuple[int, int]:
+        a = shapes.get(prefix + ".a1")
+        g = shapes.get(prefix + ".g1")
+        return (int(a[0]) if a else int(m.get("decay_rank", 16)),
+                int(g[0]) if g else int(m.get("gate_rank", 16)))
+
+    layers = []
+    for i, lc in enumerate(config["layers"]):
+        kind = lc["type"]
+        m = lc["mixer"]
+        if kind == "channel_delta":
+            mixer: MixerSpec = _delta_from_config(m, ranks(f"l{i}.mix", m))
+        elif kind == "parallel":
+            mixer = ParallelMixerSpec(
+                left=_attn_from_config(m["left"]),
+                right=_delta_from_config(
+                    m["right"], ranks(f"l{i}.mix.right", m["right"])),
+                left_scale=float(m["left_scale"]),
+                right_scale=float(m["right_scale"]))
+        else:
+            raise ValueError(f"unknown layer type {kind!r} in layer {i}")
+        mlp = lc.get("mlp")
+        if mlp is not None and mlp.get("kind", "dense") != "dense":
+            raise ValueError(f"unknown feed-forward kind {mlp['kind']!r}")
+        layers.append(HybridLayerSpec(kind=kind, mixer=mixer,
+                                      ff=int(mlp["ff"]) if mlp else 0))
+    return HybridSpec(name=name, arch="vodinex",
+                      hidden_size=int(config["width"]),
+                      vocab_size=int(config["vocab"]),
+                      layers=tuple(layers),
+                      norm_eps=float(config["norm"]["eps"]),
+                      residual_mult=float(config["residual_mult"]),
+                      max_context=int(config.get("max_context", 1 << 20)),
+                      checkpoint_dir=checkpoint_dir)

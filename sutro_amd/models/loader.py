@@ -58,8 +58,53 @@ def _shard_slice(p: torch.nn.Parameter, full: torch.Tensor) -> torch.Tensor:
     return torch.cat(parts, dim=dim)
 
 
+def _load_by_targets(model: torch.nn.Module, path: str, strict: bool) -> int:
+    """Models that publish `checkpoint_targets()` (checkpoint tensor name ->
+    (parameter, dim, start, length, scale)) are filled section by section:
+    the tensor, times `scale`, lands in parameter.narrow(dim, start, length);
+    dim None means a 0-d tensor. Every target must be met exactly once."""
+    params: Dict[str, torch.nn.Parameter] = dict(model.named_parameters())
+    targets = model.checkpoint_targets()
+    seen = set()
+    unexpected: List[str] = []
+    for name, tensor in _iter_safetensors(path):
+        tgt = targets.get(name)
+        if tgt is None:
+            unexpected.append(name)
+            continue
+        pname, dim, start, length, scale = tgt
+        p = params[pname]
+        src = tensor.to(torch.float32)
+        if scale != 1.0:
+            src = src * scale
+        with torch.no_grad():
+            if dim is None:
+                if src.numel() != 1:
+                    raise ValueError(f"{name}: expected one number, got "
+                                     f"{tuple(tensor.shape)}")
+                p.copy_(src.reshape(()).to(p.dtype))
+            else:
+                dst = p.narrow(dim, start, length)
+                if tuple(dst.shape) != tuple(src.shape):
+                    raise ValueError(
+                        f"shape mismatch for {name}: checkpoint "
+                        f"{tuple(src.shape)} vs section {tuple(dst.shape)} of "
+                        f"{pname}")
+                dst.copy_(src.to(p.dtype))
+        seen.add(name)
+    missing = sorted(set(targets) - seen)
+    if strict and unexpected:
+        raise ValueError(f"checkpoint has {len(unexpected)} tensors that map "
+                         f"to no parameter: {unexpected[:6]}")
+    if strict and missing:
+        raise ValueError(f"checkpoint missing tensors: {missing[:8]}")
+    return len(seen)
+
+
 def load_weights(model: torch.nn.Module, path: str, strict: bool = True) -> int:
     """Fill `model` from a safetensors dir. Returns #parameters loaded."""
+    if hasattr(model, "checkpoint_targets"):
+        return _load_by_targets(model, path, strict)
     params: Dict[str, torch.nn.Parameter] = dict(model.named_parameters())
     pending_merge: Dict[str, Dict[str, torch.Tensor]] = {}
     loaded = set()

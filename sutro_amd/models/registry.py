@@ -14,7 +14,7 @@ HIP kernels covers the whole registry.
 from __future__ import annotations
 
 from dataclasses import dataclass, replace
-from typing import Dict
+from typing import Dict, Optional
 
 
 @dataclass(frozen=True)
@@ -42,6 +42,8 @@ class ModelSpec:
     embedding: bool = False        # embedding models: mean-pool + L2 normalize, no decode
     # parallelism default
     recommended_tp: int = 1
+    # checkpoint directory this spec was read from (None = random init)
+    checkpoint_dir: Optional[str] = None
 
     @property
     def q_size(self) -> int:
@@ -154,10 +156,101 @@ for _name in ("gpt-oss-20b", "gpt-oss-120b"):
 MODEL_REGISTRY: Dict[str, ModelSpec] = dict(_BASE)
 
 
-def get_model_spec(name: str) -> ModelSpec:
-    """Resolve a model name to its spec. Unknown names raise KeyError with the
-    available options (the reference accepts `| str` for Functions; the engine
-    must know the architecture, so unknown names fail loudly here)."""
+def safetensors_shapes(path: str) -> Dict[str, tuple]:
+    """Tensor name -> shape for every .safetensors file under `path`, read
+    from the files' JSON headers only (8-byte little-endian header length,
+    then the header); no tensor data is touched."""
+    import json
+    import os
+    import struct
+
+    shapes: Dict[str, tuple] = {}
+    for fn in sorted(os.listdir(path)):
+        if not fn.endswith(".safetensors"):
+            continue
+        with open(os.path.join(path, fn), "rb") as f:
+            (n,) = struct.unpack("<Q", f.read(8))
+            header = json.loads(f.read(n))
+        for k, v in header.items():
+            if k != "__metadata__":
+                shapes[k] = tuple(v["shape"])
+    return shapes
+
+
+def spec_from_dir(path: str, name: Optional[str] = None):
+    """Spec of a checkpoint directory, chosen by its ``config.json``.
+
+    ``"architecture": "Vodinex"`` gives a layer-list :class:`HybridSpec`;
+    a Hugging-Face style ``"architectures": ["Qwen3...ForCausalLM"]`` gives a
+    :class:`ModelSpec` of the Qwen3 family. The returned spec remembers the
+    directory, so engines built from it load its weights."""
+    import json
+    import os
+
+    with open(os.path.join(path, "config.json")) as f:
+        cfg = json.load(f)
+    name = name or os.path.basename(os.path.normpath(path)) or "local-model"
+    arch = cfg.get("architecture")
+    if arch is None and cfg.get("architectures"):
+        arch = cfg["architectures"][0]
+    if arch == "Vodinex":
+        from .hybrid_spec import vodinex_spec
+
+        return vodinex_spec(cfg, name=name, checkpoint_dir=path,
+                            tensor_shapes=safetensors_shapes(path))
+    if arch and arch.startswith("Qwen3"):
+        moe = int(cfg.get("num_experts", 0) or 0)
+        heads = int(cfg["num_attention_heads"])
+        return ModelSpec(
+            name=name, arch="qwen3_moe" if moe else "qwen3",
+            hidden_size=int(cfg["hidden_size"]),
+            num_layers=int(cfg["num_hidden_layers"]),
+            num_heads=heads,
+            num_kv_heads=int(cfg.get("num_key_value_heads", heads)),
+            head_dim=int(cfg.get("head_dim", cfg["hidden_size"] // heads)),
+            intermediate_size=int(cfg.get("intermediate_size", 0)),
+            vocab_size=int(cfg["vocab_size"]),
+            rope_theta=float(cfg.get("rope_theta", 1e6)),
+            rms_eps=float(cfg.get("rms_norm_eps", 1e-6)),
+            max_context=int(cfg.get("max_position_embeddings", 32768)),
+            tie_embeddings=bool(cfg.get("tie_word_embeddings", False)),
+            num_experts=moe,
+            experts_per_token=int(cfg.get("num_experts_per_tok", 0) or 0),
+            moe_intermediate_size=int(cfg.get("moe_intermediate_size", 0) or 0),
+            checkpoint_dir=path)
+    raise KeyError(f"config.json under {path!r} names no known architecture "
+                   f"({arch!r})")
+
+
+def register_model_dir(name: str, path: str):
+    """Make a local checkpoint directory servable under `name`."""
+    spec = spec_from_dir(path, name=name)
+    MODEL_REGISTRY[name] = spec
+    return spec
+
+
+def build_model(spec, dtype, max_len: int, tp=None, moe_ep: bool = False):
+    """Instantiate the model class that serves `spec.arch`."""
+    if spec.arch == "vodinex":
+        from .vodinex import VodinexModel
+
+        return VodinexModel(spec, dtype, max_len, tp)
+    from .qwen3 import Qwen3Model
+
+    return Qwen3Model(spec, dtype, max_len, tp, moe_ep=moe_ep)
+
+
+def get_model_spec(name: str):
+    """Resolve a model name to its spec. A path to a checkpoint directory
+    (holding config.json) resolves to the spec its config describes. Unknown
+    names raise KeyError with the available options (the reference accepts
+    `| str` for Functions; the engine must know the architecture, so unknown
+    names fail loudly here)."""
+    import os
+
+    if name not in MODEL_REGISTRY and os.path.isfile(
+            os.path.join(name, "config.json")):
+        return spec_from_dir(name)
     try:
         return MODEL_REGISTRY[name]
     except KeyError:

@@ -165,3 +165,221 @@ def grouped_gemm(out, a, w, row_tok, tile_off, counts, max_tiles, gate_silu,
         else:
             out[s0:s0 + c] = (rows @ w[e].T.float()).to(out.dtype)
     return out
+
+
+# --------------------------------------------------------------------------
+# Layer-list ("hybrid") decoders: scalar-gain norms, gated residuals, local
+# (chunked / windowed) attention with split key/value sizes, and the gated
+# delta rule. Projections of one sublayer arrive merged in one [T, N] buffer
+# (`proj`); ops address their sections by column offset.
+# --------------------------------------------------------------------------
+
+
+def gelu_tanh(z: torch.Tensor) -> torch.Tensor:
+    return 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z * z * z)))
+
+
+def gelu_tanh_mul(proj: torch.Tensor, gate_off: int, up_off: int, ff: int) -> torch.Tensor:
+    g = proj[:, gate_off:gate_off + ff].float()
+    u = proj[:, up_off:up_off + ff].float()
+    return (gelu_tanh(g) * u).to(proj.dtype)
+
+
+def gated_norm_residual(x: torch.Tensor, y: torch.Tensor, proj: torch.Tensor,
+                        gate_off: int, gain: torch.Tensor, eps: float,
+                        mult: float, h_out=None) -> None:
+    """x (fp32, in place) += mult * gain * n(y * sigmoid(gate)), with
+    n(z) = z / sqrt(mean(z^2) + eps) and one scalar gain for all channels;
+    h_out, when given, receives the new x in its own dtype."""
+    W = x.shape[-1]
+    z = y.float() * torch.sigmoid(proj[:, gate_off:gate_off + W].float())
+    z = z * torch.rsqrt(z.pow(2).mean(-1, keepdim=True) + eps)
+    x.add_(z * (mult * gain.float()))
+    if h_out is not None:
+        h_out.copy_(x.to(h_out.dtype))
+
+
+def scalar_rmsnorm(x: torch.Tensor, gain: torch.Tensor, eps: float,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+            * gain.float()).to(out_dtype)
+
+
+def rope_inv_freq(rot_dims: int, base: float) -> torch.Tensor:
+    """fp32 [rot_dims/2]: f_i = base^(-2i/rot_dims), rounded once from fp64."""
+    half = rot_dims // 2
+    i = torch.arange(half, dtype=torch.float64)
+    return (float(base) ** (-2.0 * i / max(1, rot_dims))).float()
+
+
+def attn_prep(proj, q_off, k_off, v_off, H, G, dk, dv, q_norm_w, k_norm_w,
+              eps, inv_freq, positions, slot_mapping, k_cache, v_cache):
+    """Split q/k/v sections out of `proj`, per-head RMS norm on q and k
+    (weights may be None), rotate the first 2*len(inv_freq) dims of each q/k
+    head (rotate-half pairing, fp32 angles = position * inv_freq), write k and
+    v into their paged caches and return q [T, H, dk]."""
+    T = proj.shape[0]
+    q = proj[:, q_off:q_off + H * dk].float().reshape(T, H, dk)
+    k = proj[:, k_off:k_off + G * dk].float().reshape(T, G, dk)
+    v = proj[:, v_off:v_off + G * dv].reshape(T, G, dv)
+
+    def norm(x, w):
+        if w is None:
+            return x
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+
+    q, k = norm(q, q_norm_w), norm(k, k_norm_w)
+    half = inv_freq.numel()
+    if half:
+        ang = positions.to(torch.float32).unsqueeze(1) * inv_freq.float().unsqueeze(0)
+        c, s = ang.cos().unsqueeze(1), ang.sin().unsqueeze(1)
+
+        def rot(x):
+            a, b, rest = x[..., :half], x[..., half:2 * half], x[..., 2 * half:]
+            return torch.cat([a * c - b * s, b * c + a * s, rest], -1)
+
+        q, k = rot(q), rot(k)
+    bs = k_cache.shape[2]
+    blk = slot_mapping // bs
+    off = slot_mapping % bs
+    k_cache[blk, :, off] = k.to(k_cache.dtype)
+    v_cache[blk, :, off] = v.to(v_cache.dtype)
+    return q.to(proj.dtype)
+
+
+def local_attention(q, k_cache, v_cache, block_tables, seq_lens,
+                    query_start_locs, scale, chunk, window, proj, gate_off,
+                    out, out_off, out_scale):
+    """Softmax attention of each sequence's new tokens over its cached keys
+    under a local mask: query at position i sees j <= i with
+    j >= (i // chunk) * chunk (chunk > 0) and j > i - window (window > 0).
+    Head h's result is multiplied by out_scale * sigmoid(proj[t, gate_off+h])
+    (gate_off < 0: no gate) and written to out[t, out_off + h*dv : ...]."""
+    T, H, dk = q.shape
+    G, bs, dv = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
+    rep = H // G
+    S = seq_lens.numel()
+    for s in range(S):
+        q0, q1 = int(query_start_locs[s]), int(query_start_locs[s + 1])
+        nq = q1 - q0
+        if nq == 0:
+            continue
+        L = int(seq_lens[s])
+        nblk = (L + bs - 1) // bs
+        blocks = block_tables[s, :nblk].long()
+        keys = k_cache[blocks].transpose(0, 1).reshape(G, nblk * bs, dk)[:, :L].float()
+        vals = v_cache[blocks].transpose(0, 1).reshape(G, nblk * bs, dv)[:, :L].float()
+        qs = q[q0:q1].float().transpose(0, 1)                  # [H, nq, dk]
+        kh = keys.repeat_interleave(rep, dim=0)
+        vh = vals.repeat_interleave(rep, dim=0)
+        scores = torch.einsum("hqd,hkd->hqk", qs, kh) * scale
+        kpos = torch.arange(L, device=q.device).unsqueeze(0)
+        qpos = torch.arange(L - nq, L, device=q.device).unsqueeze(1)
+        hidden = kpos > qpos
+        if chunk > 0:
+            hidden = hidden | (kpos < (qpos // chunk) * chunk)
+        if window > 0:
+            hidden = hidden | (kpos <= qpos - window)
+        scores.masked_fill_(hidden.unsqueeze(0), float("-inf"))
+        o = torch.einsum("hqk,hkd->hqd", torch.softmax(scores, dim=-1), vh)
+        o = o.transpose(0, 1) * out_scale                      # [nq, H, dv]
+        if gate_off >= 0:
+            o = o * torch.sigmoid(proj[q0:q1, gate_off:gate_off + H].float()).unsqueeze(-1)
+        out[q0:q1, out_off:out_off + H * dv] = o.reshape(nq, H * dv).to(out.dtype)
+
+
+def delta_prep(proj, q_off, k_off, v_off, b_off, a1_off, H, G, dk, dv,
+               conv_w, a2, dt_bias, a_log, conv_state, state_slots,
+               query_start_locs, seq_lens):
+    """Inputs of the gated delta rule for every new token.
+
+    q/k/v sections of `proj` pass a causal depthwise filter (`conv_w`
+    [C, taps] over channels ordered q|k|v, last tap = current token; inputs
+    before the sequence start are zero; the filter's history for a sequence
+    that continues comes from conv_state[slot] = its last taps-1 raw inputs,
+    time-major) and silu; q and k become unit vectors per head (q also times
+    dk^-1/2). beta = sigmoid(b section). decay = exp(-exp(a_log[h]) *
+    softplus(a2 @ a1 + dt_bias)) per head and key channel. conv_state is
+    brought up to date. Returns fp32 (q [T,G,dk], k [T,G,dk], v [T,H,dv],
+    decay [T,H,dk], beta [T,H])."""
+    T = proj.shape[0]
+    Cq, Cv = G * dk, H * dv
+    C = 2 * Cq + Cv
+    taps = conv_w.shape[1]
+    raw = torch.cat([proj[:, q_off:q_off + Cq], proj[:, k_off:k_off + Cq],
+                     proj[:, v_off:v_off + Cv]], dim=1).float()
+    y = torch.empty_like(raw)
+    S = seq_lens.numel()
+    wf = conv_w.float()
+    for s in range(S):
+        a, b = int(query_start_locs[s]), int(query_start_locs[s + 1])
+        n = b - a
+        if n == 0:
+            continue
+        start = int(seq_lens[s]) - n
+        slot = int(state_slots[s])
+        if taps > 1:
+            hist = (conv_state[slot].float() if start > 0
+                    else torch.zeros(taps - 1, C, dtype=torch.float32, device=proj.device))
+            ext = torch.cat([hist, raw[a:b]], dim=0)          # [taps-1+n, C]
+            conv_state[slot] = ext[-(taps - 1):].to(conv_state.dtype)
+        else:
+            ext = raw[a:b]
+        acc = torch.zeros(n, C, dtype=torch.float32, device=proj.device)
+        for j in range(taps):
+            acc = acc + ext[j:j + n] * wf[:, j]
+        y[a:b] = acc * torch.sigmoid(acc)
+    qn = y[:, :Cq].reshape(T, G, dk)
+    kn = y[:, Cq:2 * Cq].reshape(T, G, dk)
+    v = y[:, 2 * Cq:].reshape(T, H, dv).contiguous()
+    qn = qn * torch.rsqrt(qn.pow(2).sum(-1, keepdim=True) + 1e-6) * (float(dk) ** -0.5)
+    kn = kn * torch.rsqrt(kn.pow(2).sum(-1, keepdim=True) + 1e-6)
+    beta = torch.sigmoid(proj[:, b_off:b_off + H].float())
+    r = a2.shape[1]
+    a = proj[:, a1_off:a1_off + r].float() @ a2.float().T + dt_bias.float()
+    decay = torch.exp(-torch.exp(a_log.float()).view(1, H, 1)
+                      * torch.nn.functional.softplus(a).view(T, H, dk))
+    return qn.contiguous(), kn.contiguous(), v, decay.contiguous(), beta.contiguous()
+
+
+def delta_scan(qn, kn, v, decay, beta, ssm_state, state_slots,
+               query_start_locs, seq_lens):
+    """Token-by-token gated delta rule per sequence and head, state
+    ssm_state[slot] = S [H, dk, dv] (fp32, zero at a sequence's start):
+        S <- decay[:, None] * S;  u = beta * (v - S^T k);
+        S <- S + k u^T;           o = S^T q.
+    Returns o [T, H, dv] fp32 and leaves the new state in ssm_state."""
+    T, H, dv = v.shape
+    G = kn.shape[1]
+    rep = H // G
+    o = torch.empty(T, H, dv, dtype=torch.float32, device=v.device)
+    S_n = seq_lens.numel()
+    for s in range(S_n):
+        a, b = int(query_start_locs[s]), int(query_start_locs[s + 1])
+        n = b - a
+        if n == 0:
+            continue
+        start = int(seq_lens[s]) - n
+        slot = int(state_slots[s])
+        St = (ssm_state[slot].clone() if start > 0
+              else torch.zeros_like(ssm_state[slot]))
+        for t in range(a, b):
+            kt = kn[t].repeat_interleave(rep, dim=0)           # [H, dk]
+            qt = qn[t].repeat_interleave(rep, dim=0)
+            St = St * decay[t].unsqueeze(-1)
+            u = beta[t].unsqueeze(-1) * (v[t] - torch.einsum("hkv,hk->hv", St, kt))
+            St = St + kt.unsqueeze(-1) * u.unsqueeze(1)
+            o[t] = torch.einsum("hkv,hk->hv", St, qt)
+        ssm_state[slot] = St
+    return o
+
+
+def delta_out(o, norm_w, proj, g1_off, g2, eps, out, out_off, out_scale):
+    """out[t, out_off + h*dv + j] = out_scale * n(o[t,h])_j * norm_w[j] *
+    sigmoid(g2 @ g1)[h*dv + j], n = divide by the root mean square over dv."""
+    T, H, dv = o.shape
+    r = g2.shape[1]
+    gate = torch.sigmoid(proj[:, g1_off:g1_off + r].float() @ g2.float().T).view(T, H, dv)
+    y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()
+    out[:, out_off:out_off + H * dv] = (y * gate * out_scale).reshape(T, H * dv).to(out.dtype)

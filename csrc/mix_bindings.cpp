@@ -1,0 +1,303 @@
+// Python bindings of the layer-list decoder kernels (sutro_amd._C_mix).
+// Shapes and dtypes are validated here; raw pointers and the current HIP
+// stream go to the extern "C" launchers in mix_*.hip. Activation tensors are
+// bf16 or fp32 (all of one call the same); recurrence inputs, norm weights
+// and the residual stream are fp32.
+#include <torch/extension.h>
+
+#include <hip/hip_runtime.h>
+#include <c10/hip/HIPStream.h>
+
+#define CHECK_GPU(x) TORCH_CHECK((x).is_cuda(), #x " must be a GPU tensor")
+#define CHECK_CONTIG(x) TORCH_CHECK((x).is_contiguous(), #x " must be contiguous")
+#define CHECK_F32(x) \
+  TORCH_CHECK((x).scalar_type() == at::kFloat, #x " must be fp32")
+#define CHECK_I32(x) \
+  TORCH_CHECK((x).scalar_type() == at::kInt, #x " must be int32")
+#define CHECK_I64(x) \
+  TORCH_CHECK((x).scalar_type() == at::kLong, #x " must be int64")
+
+static hipStream_t cur_stream() {
+  return c10::hip::getCurrentHIPStream().stream();
+}
+
+// 1 = fp32 activations, 0 = bf16
+static int act_kind(const torch::Tensor& t) {
+  TORCH_CHECK(t.scalar_type() == at::kFloat || t.scalar_type() == at::kBFloat16,
+              "activations must be bf16 or fp32");
+  return t.scalar_type() == at::kFloat ? 1 : 0;
+}
+
+static void check_proj(const torch::Tensor& proj, long off, long width,
+                       const char* what) {
+  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1, "proj must be [T, N] rows");
+  TORCH_CHECK(off >= 0 && off + width <= proj.size(1), what,
+              " section outside the projection buffer");
+}
+
+extern "C" {
+void mix_gelu_tanh_mul(void*, const void*, long, int, int, long, int, int,
+                       hipStream_t);
+void mix_gated_norm_residual(float*, const void*, const void*, long, int,
+                             const float*, float, float, void*, long, int, int,
+                             hipStream_t);
+void mix_scalar_rmsnorm(void*, const float*, const float*, float, long, int,
+                        int, hipStream_t);
+void mix_attn_prep(void*, const void*, long, int, int, int, const float*,
+                   const float*, float, const float*, int, const long*,
+                   const long*, void*, void*, long, int, int, int, int, int,
+                   int, hipStream_t);
+void mix_local_attention(void*, long, int, const void*, const void*,
+                         const void*, const int*, int, const int*, const int*,
+                         const int*, float, int, int, const void*, long, int,
+                         float, long, int, int, int, int, int, int,
+                         hipStream_t);
+void mix_delta_prep(float*, float*, float*, float*, float*, const void*, long,
+                    int, int, int, int, int, const float*, int, const float*,
+                    int, const float*, const float*, float*, const int*,
+                    const int*, const int*, const int*, long, int, int, int,
+                    int, int, int, hipStream_t);
+void mix_delta_scan(float*, const float*, const float*, const float*,
+                    const float*, const float*, float*, const int*, const int*,
+                    const int*, int, int, int, int, int, hipStream_t);
+void mix_delta_out(void*, long, int, const float*, const float*, const void*,
+                   long, int, const float*, int, float, float, long, int, int,
+                   int, hipStream_t);
+}
+
+void gelu_tanh_mul(torch::Tensor out, torch::Tensor proj, long gate_off,
+                   long up_off) {
+  CHECK_GPU(proj); CHECK_GPU(out); CHECK_CONTIG(out);
+  const long T = out.size(0), F = out.size(1);
+  TORCH_CHECK(out.scalar_type() == proj.scalar_type(), "dtype mismatch");
+  check_proj(proj, gate_off, F, "gate");
+  check_proj(proj, up_off, F, "up");
+  TORCH_CHECK(proj.size(0) == T, "row mismatch");
+  mix_gelu_tanh_mul(out.data_ptr(), proj.data_ptr(), proj.stride(0),
+                    (int)gate_off, (int)up_off, T, (int)F, act_kind(proj),
+                    cur_stream());
+}
+
+void gated_norm_residual(torch::Tensor x, torch::Tensor y, torch::Tensor proj,
+                         long gate_off, torch::Tensor gain, double eps,
+                         double mult, c10::optional<torch::Tensor> h_out) {
+  CHECK_GPU(x); CHECK_CONTIG(x); CHECK_F32(x);
+  CHECK_GPU(y); CHECK_CONTIG(y); CHECK_GPU(gain); CHECK_F32(gain);
+  const long T = x.size(0), W = x.size(1);
+  TORCH_CHECK(y.size(0) == T && y.size(1) == W, "y shape");
+  TORCH_CHECK(y.scalar_type() == proj.scalar_type(), "dtype mismatch");
+  TORCH_CHECK(proj.size(0) == T, "row mismatch");
+  check_proj(proj, gate_off, W, "gate");
+  void* hp = nullptr;
+  if (h_out.has_value()) {
+    CHECK_CONTIG(*h_out);
+    TORCH_CHECK(h_out->scalar_type() == y.scalar_type() &&
+                h_out->size(0) == T && h_out->size(1) == W, "h_out shape");
+    hp = h_out->data_ptr();
+  }
+  mix_gated_norm_residual(x.data_ptr<float>(), y.data_ptr(), proj.data_ptr(),
+                          proj.stride(0), (int)gate_off,
+                          gain.data_ptr<float>(), (float)eps, (float)mult, hp,
+                          T, (int)W, act_kind(y), cur_stream());
+}
+
+void scalar_rmsnorm(torch::Tensor out, torch::Tensor x, torch::Tensor gain,
+                    double eps) {
+  CHECK_GPU(x); CHECK_CONTIG(x); CHECK_F32(x); CHECK_CONTIG(out);
+  CHECK_GPU(gain); CHECK_F32(gain);
+  const long W = x.size(-1), T = x.numel() / W;
+  TORCH_CHECK(out.numel() == x.numel(), "out shape");
+  mix_scalar_rmsnorm(out.data_ptr(), x.data_ptr<float>(),
+                     gain.data_ptr<float>(), (float)eps, T, (int)W,
+                     act_kind(out), cur_stream());
+}
+
+void attn_prep(torch::Tensor q_out, torch::Tensor proj, long q_off, long k_off,
+               long v_off, c10::optional<torch::Tensor> q_w,
+               c10::optional<torch::Tensor> k_w, double eps,
+               torch::Tensor inv_freq, torch::Tensor positions,
+               torch::Tensor slots, torch::Tensor k_cache,
+               torch::Tensor v_cache) {
+  CHECK_GPU(proj); CHECK_GPU(q_out); CHECK_CONTIG(q_out);
+  CHECK_CONTIG(k_cache); CHECK_CONTIG(v_cache);
+  CHECK_I64(positions); CHECK_I64(slots); CHECK_F32(inv_freq);
+  CHECK_CONTIG(inv_freq);
+  const long T = q_out.size(0), H = q_out.size(1), dk = q_out.size(2);
+  const long G = k_cache.size(1), page = k_cache.size(2);
+  const long dv = v_cache.size(3);
+  TORCH_CHECK(k_cache.size(3) == dk && v_cache.size(1) == G &&
+              v_cache.size(2) == page, "cache shapes");
+  TORCH_CHECK(q_out.scalar_type() == proj.scalar_type() &&
+              k_cache.scalar_type() == proj.scalar_type() &&
+              v_cache.scalar_type() == proj.scalar_type(),
+              "q, caches and projections must share one dtype");
+  TORCH_CHECK(proj.size(0) == T && positions.numel() == T &&
+              slots.numel() == T, "row mismatch");
+  check_proj(proj, q_off, H * dk, "q");
+  check_proj(proj, k_off, G * dk, "k");
+  check_proj(proj, v_off, G * dv, "v");
+  const long half = inv_freq.numel();
+  TORCH_CHECK(2 * half <= dk, "rotated prefix longer than the head");
+  const float* qw = nullptr; const float* kw = nullptr;
+  if (q_w.has_value()) {
+    CHECK_F32(*q_w); TORCH_CHECK(q_w->numel() == dk, "q norm size");
+    qw = q_w->data_ptr<float>();
+  }
+  if (k_w.has_value()) {
+    CHECK_F32(*k_w); TORCH_CHECK(k_w->numel() == dk, "k norm size");
+    kw = k_w->data_ptr<float>();
+  }
+  mix_attn_prep(q_out.data_ptr(), proj.data_ptr(), proj.stride(0), (int)q_off,
+                (int)k_off, (int)v_off, qw, kw, (float)eps,
+                inv_freq.data_ptr<float>(), (int)half,
+                positions.data_ptr<long>(), slots.data_ptr<long>(),
+                k_cache.data_ptr(), v_cache.data_ptr(), T, (int)H, (int)G,
+                (int)dk, (int)dv, (int)page, act_kind(proj), cur_stream());
+}
+
+void local_attention(torch::Tensor out, long out_off, torch::Tensor q,
+                     torch::Tensor k_cache, torch::Tensor v_cache,
+                     torch::Tensor bt, torch::Tensor seq_lens,
+                     torch::Tensor qlocs, torch::Tensor token_seq,
+                     double scale, long chunk, long window, torch::Tensor proj,
+                     long gate_off, double out_scale) {
+  CHECK_GPU(q); CHECK_CONTIG(q); CHECK_CONTIG(k_cache); CHECK_CONTIG(v_cache);
+  CHECK_I32(bt); CHECK_I32(seq_lens); CHECK_I32(qlocs); CHECK_I32(token_seq);
+  CHECK_CONTIG(bt);
+  const long T = q.size(0), H = q.size(1), dk = q.size(2);
+  const long G = k_cache.size(1), page = k_cache.size(2);
+  const long dv = v_cache.size(3);
+  TORCH_CHECK(k_cache.size(3) == dk, "key size mismatch");
+  TORCH_CHECK(H % G == 0, "heads must be a multiple of kv heads");
+  TORCH_CHECK(dv <= 256 && dk <= 4096, "unsupported head sizes");
+  TORCH_CHECK(out.dim() == 2 && out.stride(1) == 1 && out.size(0) == T &&
+              out_off >= 0 && out_off + H * dv <= out.size(1), "out section");
+  TORCH_CHECK(out.scalar_type() == q.scalar_type() &&
+              k_cache.scalar_type() == q.scalar_type() &&
+              v_cache.scalar_type() == q.scalar_type() &&
+              proj.scalar_type() == q.scalar_type(), "dtype mismatch");
+  TORCH_CHECK(token_seq.numel() == T && qlocs.numel() == seq_lens.numel() + 1 &&
+              bt.size(0) == seq_lens.numel(), "batch metadata sizes");
+  if (gate_off >= 0) check_proj(proj, gate_off, H, "gate");
+  TORCH_CHECK(proj.size(0) == T, "row mismatch");
+  mix_local_attention(out.data_ptr(), out.stride(0), (int)out_off,
+                      q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                      bt.data_ptr<int>(), (int)bt.size(1),
+                      seq_lens.data_ptr<int>(), qlocs.data_ptr<int>(),
+                      token_seq.data_ptr<int>(), (float)scale, (int)chunk,
+                      (int)window, proj.data_ptr(), proj.stride(0),
+                      (int)gate_off, (float)out_scale, T, (int)H, (int)G,
+                      (int)dk, (int)dv, (int)page, act_kind(q), cur_stream());
+}
+
+void delta_prep(torch::Tensor qn, torch::Tensor kn, torch::Tensor v,
+                torch::Tensor decay, torch::Tensor beta, torch::Tensor proj,
+                long q_off, long k_off, long v_off, long b_off, long a1_off,
+                torch::Tensor conv_w, torch::Tensor a2, torch::Tensor dt_bias,
+                torch::Tensor a_log, torch::Tensor conv_state,
+                torch::Tensor state_slots, torch::Tensor qlocs,
+                torch::Tensor seq_lens, torch::Tensor token_seq) {
+  CHECK_GPU(proj);
+  CHECK_F32(qn); CHECK_F32(kn); CHECK_F32(v); CHECK_F32(decay); CHECK_F32(beta);
+  CHECK_CONTIG(qn); CHECK_CONTIG(kn); CHECK_CONTIG(v); CHECK_CONTIG(decay);
+  CHECK_CONTIG(beta);
+  CHECK_F32(conv_w); CHECK_F32(a2); CHECK_F32(dt_bias); CHECK_F32(a_log);
+  CHECK_F32(conv_state); CHECK_CONTIG(conv_w); CHECK_CONTIG(a2);
+  CHECK_CONTIG(conv_state);
+  CHECK_I32(state_slots); CHECK_I32(qlocs); CHECK_I32(seq_lens);
+  CHECK_I32(token_seq);
+  const long T = v.size(0), H = v.size(1), dv = v.size(2);
+  const long G = qn.size(1), dk = qn.size(2);
+  const long S = seq_lens.numel();
+  const long C = 2 * G * dk + H * dv, taps = conv_w.size(1);
+  const long rank = a2.size(1);
+  TORCH_CHECK(dk <= 256 && dv <= 256, "head sizes above 256 are unsupported");
+  TORCH_CHECK(H % G == 0, "heads must be a multiple of kv heads");
+  TORCH_CHECK(conv_w.size(0) == C, "filter channels");
+  TORCH_CHECK(a2.size(0) == H * dk && dt_bias.numel() == H * dk &&
+              a_log.numel() == H, "decay parameter sizes");
+  TORCH_CHECK(conv_state.dim() == 3 && conv_state.size(2) == C &&
+              conv_state.size(1) >= taps - 1 &&
+              (taps == 1 || conv_state.size(1) == taps - 1),
+              "filter state shape");
+  TORCH_CHECK(proj.size(0) == T && token_seq.numel() == T &&
+              qlocs.numel() == S + 1 && state_slots.numel() == S &&
+              kn.size(0) == T && decay.size(0) == T && beta.size(0) == T,
+              "batch metadata sizes");
+  check_proj(proj, q_off, G * dk, "q");
+  check_proj(proj, k_off, G * dk, "k");
+  check_proj(proj, v_off, H * dv, "v");
+  check_proj(proj, b_off, H, "beta");
+  check_proj(proj, a1_off, rank, "decay input");
+  mix_delta_prep(qn.data_ptr<float>(), kn.data_ptr<float>(),
+                 v.data_ptr<float>(), decay.data_ptr<float>(),
+                 beta.data_ptr<float>(), proj.data_ptr(), proj.stride(0),
+                 (int)q_off, (int)k_off, (int)v_off, (int)b_off, (int)a1_off,
+                 conv_w.data_ptr<float>(), (int)taps, a2.data_ptr<float>(),
+                 (int)rank, dt_bias.data_ptr<float>(), a_log.data_ptr<float>(),
+                 conv_state.data_ptr<float>(), state_slots.data_ptr<int>(),
+                 qlocs.data_ptr<int>(), seq_lens.data_ptr<int>(),
+                 token_seq.data_ptr<int>(), T, (int)S, (int)H, (int)G, (int)dk,
+                 (int)dv, act_kind(proj), cur_stream());
+}
+
+void delta_scan(torch::Tensor o, torch::Tensor qn, torch::Tensor kn,
+                torch::Tensor v, torch::Tensor decay, torch::Tensor beta,
+                torch::Tensor ssm, torch::Tensor state_slots,
+                torch::Tensor qlocs, torch::Tensor seq_lens) {
+  CHECK_GPU(v); CHECK_F32(o); CHECK_F32(qn); CHECK_F32(kn); CHECK_F32(v);
+  CHECK_F32(decay); CHECK_F32(beta); CHECK_F32(ssm);
+  CHECK_CONTIG(o); CHECK_CONTIG(qn); CHECK_CONTIG(kn); CHECK_CONTIG(v);
+  CHECK_CONTIG(decay); CHECK_CONTIG(beta); CHECK_CONTIG(ssm);
+  CHECK_I32(state_slots); CHECK_I32(qlocs); CHECK_I32(seq_lens);
+  const long T = v.size(0), H = v.size(1), dv = v.size(2);
+  const long G = kn.size(1), dk = kn.size(2);
+  const long S = seq_lens.numel();
+  TORCH_CHECK(dk <= 256, "key size above 256 is unsupported");
+  TORCH_CHECK(H % G == 0, "heads must be a multiple of kv heads");
+  TORCH_CHECK(ssm.dim() == 4 && ssm.size(1) == H && ssm.size(2) == dk &&
+              ssm.size(3) == dv, "state shape");
+  TORCH_CHECK(o.numel() == v.numel() && qn.numel() == kn.numel() &&
+              kn.size(0) == T && decay.numel() == T * H * dk &&
+              beta.numel() == T * H && qlocs.numel() == S + 1 &&
+              state_slots.numel() == S, "operand sizes");
+  mix_delta_scan(o.data_ptr<float>(), qn.data_ptr<float>(),
+                 kn.data_ptr<float>(), v.data_ptr<float>(),
+                 decay.data_ptr<float>(), beta.data_ptr<float>(),
+                 ssm.data_ptr<float>(), state_slots.data_ptr<int>(),
+                 qlocs.data_ptr<int>(), seq_lens.data_ptr<int>(), (int)S,
+                 (int)H, (int)G, (int)dk, (int)dv, cur_stream());
+}
+
+void delta_out(torch::Tensor out, long out_off, torch::Tensor o,
+               torch::Tensor norm_w, torch::Tensor proj, long g1_off,
+               torch::Tensor g2, double eps, double out_scale) {
+  CHECK_GPU(o); CHECK_F32(o); CHECK_CONTIG(o); CHECK_F32(norm_w);
+  CHECK_F32(g2); CHECK_CONTIG(g2);
+  const long T = o.size(0), H = o.size(1), dv = o.size(2);
+  const long rank = g2.size(1);
+  TORCH_CHECK(norm_w.numel() == dv && g2.size(0) == H * dv, "parameter sizes");
+  TORCH_CHECK(out.dim() == 2 && out.stride(1) == 1 && out.size(0) == T &&
+              out_off >= 0 && out_off + H * dv <= out.size(1), "out section");
+  TORCH_CHECK(out.scalar_type() == proj.scalar_type(), "dtype mismatch");
+  TORCH_CHECK(proj.size(0) == T, "row mismatch");
+  check_proj(proj, g1_off, rank, "gate input");
+  mix_delta_out(out.data_ptr(), out.stride(0), (int)out_off,
+                o.data_ptr<float>(), norm_w.data_ptr<float>(), proj.data_ptr(),
+                proj.stride(0), (int)g1_off, g2.data_ptr<float>(), (int)rank,
+                (float)eps, (float)out_scale, T, (int)H, (int)dv,
+                act_kind(out), cur_stream());
+}
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("gelu_tanh_mul", &gelu_tanh_mul, "tanh-GELU(gate) * up");
+  m.def("gated_norm_residual", &gated_norm_residual,
+        "x += m * g * n(y * sigmoid(gate)); h = cast(x)");
+  m.def("scalar_rmsnorm", &scalar_rmsnorm, "RMS norm with one scalar gain");
+  m.def("attn_prep", &attn_prep, "q/k norm + partial rotation + paged K/V write");
+  m.def("local_attention", &local_attention,
+        "chunked/windowed paged attention with per-head output gate");
+  m.def("delta_prep", &delta_prep, "delta-rule inputs: filters, norms, gates");
+  m.def("delta_scan", &delta_scan, "gated delta rule over new tokens");
+  m.def("delta_out", &delta_out, "per-head norm + low-rank gate of the read-out");
+}

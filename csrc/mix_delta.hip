@@ -1,0 +1,298 @@
+// Gated delta rule with one decay per head and key channel.
+//
+//   delta_prep         short causal depthwise filter + silu on the q|k|v
+//                      channels, unit-norm q (times dk^-1/2) and k, beta =
+//                      sigmoid, decay = exp(-exp(A_log) * softplus(a2 a1 + dt))
+//   conv_state_update  keeps the last taps-1 raw filter inputs per sequence
+//   delta_scan         S <- decay * S; u = beta (v - S^T k); S <- S + k u^T;
+//                      o = S^T q, token by token, S [dk, dv] fp32 per head
+//   delta_out          o / rms(o) * w * sigmoid(g2 g1), cast, into the
+//                      output-projection input
+//
+// Everything the recurrence consumes is fp32. A sequence whose first token
+// (position 0) is in the batch starts from zero filter history and zero S,
+// whatever its state slot held before.
+//
+// delta_scan maps the state onto lanes by COLUMN: the dv columns of S never
+// interact, so a column is owned by R adjacent lanes holding dk/R rows each
+// in registers; one token costs two R-lane shuffle reductions and no LDS
+// traffic or barriers. Blocks cover (sequence, head, group of columns).
+#include "mix_common.h"
+
+#define WPB 4
+
+// merged channel c (q | k | v order) -> column of the projection buffer
+__device__ __forceinline__ int chan_col(int c, int Cq, int q_off, int k_off,
+                                        int v_off) {
+  return c < Cq ? q_off + c : (c < 2 * Cq ? k_off + c - Cq : v_off + c - 2 * Cq);
+}
+
+template <typename A>
+__global__ void delta_prep_kernel(
+    float* __restrict__ qn, float* __restrict__ kn, float* __restrict__ vv,
+    float* __restrict__ decay, float* __restrict__ beta,
+    const A* __restrict__ proj, long ld, int q_off, int k_off, int v_off,
+    int b_off, int a1_off, const float* __restrict__ conv_w, int taps,
+    const float* __restrict__ a2, int rank, const float* __restrict__ dt_bias,
+    const float* __restrict__ a_log, const float* __restrict__ conv_state,
+    const int* __restrict__ state_slots, const int* __restrict__ qlocs,
+    const int* __restrict__ seq_lens, const int* __restrict__ token_seq,
+    long T, int H, int G, int dk, int dv) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int wid = threadIdx.x / WAVE;
+  const int units = 2 * G + 2 * H;
+  const long u = (long)blockIdx.x * WPB + wid;
+  if (u >= T * units) return;
+  const long t = u / units;
+  const int j = (int)(u - t * units);
+  const int Cq = G * dk, C = 2 * Cq + H * dv;
+
+  if (j >= 2 * G + H) {  // decay + beta of head h
+    const int h = j - 2 * G - H;
+    const A* a1 = proj + t * ld + a1_off;
+    const float rate = expf(a_log[h]);
+    for (int i = lane; i < dk; i += WAVE) {
+      const float* w = a2 + ((long)h * dk + i) * rank;
+      float a = dt_bias[h * dk + i];
+      for (int r = 0; r < rank; ++r) a += w[r] * ldf<A>(a1 + r);
+      decay[(t * H + h) * (long)dk + i] = expf(-rate * softplus_f(a));
+    }
+    if (lane == 0)
+      beta[t * H + h] = sigmoid_f(ldf<A>(proj + t * ld + b_off + h));
+    return;
+  }
+
+  // filter + silu of one q, k or v head
+  const int kind = j < G ? 0 : (j < 2 * G ? 1 : 2);
+  const int head = kind == 0 ? j : (kind == 1 ? j - G : j - 2 * G);
+  const int d = kind == 2 ? dv : dk;
+  const int c0 = (kind == 0 ? 0 : (kind == 1 ? Cq : 2 * Cq)) + head * d;
+  const int s = token_seq[t];
+  const int q0 = qlocs[s], n = qlocs[s + 1] - q0;
+  const int start = seq_lens[s] - n;      // position of the chunk's first token
+  const int jl = (int)t - q0;             // local index in the chunk
+  const float* hist = conv_state + (long)state_slots[s] * (taps - 1) * C;
+
+  float y[4];  // d <= 256
+  float ssq = 0.f;
+  int k = 0;
+  for (int i = lane; i < d; i += WAVE, ++k) {
+    const int c = c0 + i;
+    const int col = chan_col(c, Cq, q_off, k_off, v_off);
+    float acc = 0.f;
+    for (int back = 0; back < taps; ++back) {
+      float x = 0.f;
+      if (jl - back >= 0)
+        x = ldf<A>(proj + (t - back) * ld + col);
+      else if (start > 0)  // start + jl - back >= 0 is implied: the history
+        x = hist[(long)(taps - 1 - back + jl) * C + c];  // holds zeros there
+      acc += conv_w[(long)c * taps + (taps - 1 - back)] * x;
+    }
+    const float a = acc * sigmoid_f(acc);
+    y[k] = a;
+    ssq += a * a;
+  }
+  ssq = wave_sum_f32(ssq);
+  float f = 1.f;
+  if (kind != 2) {
+    f = 1.f / sqrtf(ssq + 1e-6f);
+    if (kind == 0) f *= 1.f / sqrtf((float)dk);
+  }
+  float* dst = kind == 0 ? qn + (t * G + head) * (long)dk
+                         : (kind == 1 ? kn + (t * G + head) * (long)dk
+                                      : vv + (t * H + head) * (long)dv);
+  k = 0;
+  for (int i = lane; i < d; i += WAVE, ++k) dst[i] = y[k] * f;
+}
+
+// one thread per (sequence, channel): new history = last taps-1 raw inputs
+template <typename A>
+__global__ void conv_state_update_kernel(
+    float* __restrict__ conv_state, const A* __restrict__ proj, long ld,
+    int q_off, int k_off, int v_off, int taps,
+    const int* __restrict__ state_slots, const int* __restrict__ qlocs,
+    const int* __restrict__ seq_lens, int S, int Cq, int C) {
+  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long)S * C) return;
+  const int s = (int)(idx / C), c = (int)(idx - (long)s * C);
+  const int q0 = qlocs[s], n = qlocs[s + 1] - q0;
+  if (n <= 0) return;
+  const int start = seq_lens[s] - n;
+  const int col = chan_col(c, Cq, q_off, k_off, v_off);
+  float* hist = conv_state + (long)state_slots[s] * (taps - 1) * C + c;
+  for (int i = 0; i < taps - 1; ++i) {
+    const int tau = n - (taps - 1) + i;  // chunk-local time of history row i
+    float x = 0.f;
+    if (tau >= 0)
+      x = ldf<A>(proj + (long)(q0 + tau) * ld + col);
+    else if (start > 0 && i + n <= taps - 2)
+      x = hist[(long)(i + n) * C];       // read before row i+n is rewritten
+    hist[(long)i * C] = x;
+  }
+}
+
+#define RPT 32  // state rows per lane
+
+__global__ void delta_scan_kernel(
+    float* __restrict__ o, const float* __restrict__ qn,
+    const float* __restrict__ kn, const float* __restrict__ vv,
+    const float* __restrict__ decay, const float* __restrict__ beta,
+    float* __restrict__ ssm, const int* __restrict__ state_slots,
+    const int* __restrict__ qlocs, const int* __restrict__ seq_lens, int H,
+    int G, int dk, int dv, int R, int col_groups) {
+  const int cols_pb = blockDim.x / R;
+  int b = blockIdx.x;
+  const int cg = b % col_groups; b /= col_groups;
+  const int h = b % H;
+  const int s = b / H;
+  const int r = threadIdx.x % R;
+  const int col = cg * cols_pb + threadIdx.x / R;
+  const bool cv = col < dv;
+  const int g = h / (H / G);
+  const int q0 = qlocs[s], q1 = qlocs[s + 1];
+  if (q1 <= q0) return;
+  const int start = seq_lens[s] - (q1 - q0);
+  const int i0 = r * RPT;
+  float* Sg = ssm + (((long)state_slots[s] * H + h) * dk) * dv;
+
+  float S[RPT];
+#pragma unroll
+  for (int i = 0; i < RPT; ++i)
+    S[i] = (start > 0 && cv && i0 + i < dk) ? Sg[(long)(i0 + i) * dv + col]
+                                            : 0.f;
+
+  for (int t = q0; t < q1; ++t) {
+    const float* kt = kn + ((long)t * G + g) * dk + i0;
+    const float* qt = qn + ((long)t * G + g) * dk + i0;
+    const float* dt = decay + ((long)t * H + h) * dk + i0;
+    const float vt = cv ? vv[((long)t * H + h) * dv + col] : 0.f;
+    const float bt = beta[(long)t * H + h];
+    float kk[RPT];
+    float dot = 0.f;
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+      const bool in = i0 + i < dk;
+      kk[i] = in ? kt[i] : 0.f;
+      S[i] *= in ? dt[i] : 1.f;
+      dot += S[i] * kk[i];
+    }
+    for (int off = R >> 1; off > 0; off >>= 1) dot += __shfl_xor(dot, off, WAVE);
+    const float uu = bt * (vt - dot);
+    float out = 0.f;
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+      S[i] += kk[i] * uu;
+      out += S[i] * (i0 + i < dk ? qt[i] : 0.f);
+    }
+    for (int off = R >> 1; off > 0; off >>= 1) out += __shfl_xor(out, off, WAVE);
+    if (r == 0 && cv) o[((long)t * H + h) * dv + col] = out;
+  }
+  if (cv) {
+#pragma unroll
+    for (int i = 0; i < RPT; ++i)
+      if (i0 + i < dk) Sg[(long)(i0 + i) * dv + col] = S[i];
+  }
+}
+
+template <typename A>
+__global__ void delta_out_kernel(A* __restrict__ out, long ldo, int out_off,
+                                 const float* __restrict__ o,
+                                 const float* __restrict__ norm_w,
+                                 const A* __restrict__ proj, long ld,
+                                 int g1_off, const float* __restrict__ g2,
+                                 int rank, float eps, float out_scale, long T,
+                                 int H, int dv) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const long u = (long)blockIdx.x * WPB + threadIdx.x / WAVE;
+  if (u >= T * H) return;
+  const long t = u / H;
+  const int h = (int)(u - t * H);
+  const float* orow = o + u * dv;
+  float ssq = 0.f;
+  for (int c = lane; c < dv; c += WAVE) ssq += orow[c] * orow[c];
+  ssq = wave_sum_f32(ssq);
+  const float inv = out_scale / sqrtf(ssq / (float)dv + eps);
+  const A* g1 = proj + t * ld + g1_off;
+  for (int c = lane; c < dv; c += WAVE) {
+    const float* w = g2 + ((long)h * dv + c) * rank;
+    float a = 0.f;
+    for (int r = 0; r < rank; ++r) a += w[r] * ldf<A>(g1 + r);
+    stf<A>(out + t * ldo + out_off + (long)h * dv + c,
+           orow[c] * inv * norm_w[c] * sigmoid_f(a));
+  }
+}
+
+extern "C" void mix_delta_prep(
+    float* qn, float* kn, float* vv, float* decay, float* beta,
+    const void* proj, long ld, int q_off, int k_off, int v_off, int b_off,
+    int a1_off, const float* conv_w, int taps, const float* a2, int rank,
+    const float* dt_bias, const float* a_log, float* conv_state,
+    const int* state_slots, const int* qlocs, const int* seq_lens,
+    const int* token_seq, long T, int S, int H, int G, int dk, int dv, int f32,
+    hipStream_t s) {
+  const long units = T * (2 * G + 2 * H);
+  const int grid = (int)((units + WPB - 1) / WPB);
+  if (grid == 0) return;
+  const int Cq = G * dk, C = 2 * Cq + H * dv;
+  const long su = (long)S * C;
+  const int sgrid = (int)((su + 255) / 256);
+  if (f32) {
+    hipLaunchKernelGGL(delta_prep_kernel<float>, dim3(grid), dim3(WPB * WAVE),
+                       0, s, qn, kn, vv, decay, beta, (const float*)proj, ld,
+                       q_off, k_off, v_off, b_off, a1_off, conv_w, taps, a2,
+                       rank, dt_bias, a_log, conv_state, state_slots, qlocs,
+                       seq_lens, token_seq, T, H, G, dk, dv);
+    if (taps > 1)
+      hipLaunchKernelGGL(conv_state_update_kernel<float>, dim3(sgrid),
+                         dim3(256), 0, s, conv_state, (const float*)proj, ld,
+                         q_off, k_off, v_off, taps, state_slots, qlocs,
+                         seq_lens, S, Cq, C);
+  } else {
+    hipLaunchKernelGGL(delta_prep_kernel<u16>, dim3(grid), dim3(WPB * WAVE), 0,
+                       s, qn, kn, vv, decay, beta, (const u16*)proj, ld, q_off,
+                       k_off, v_off, b_off, a1_off, conv_w, taps, a2, rank,
+                       dt_bias, a_log, conv_state, state_slots, qlocs,
+                       seq_lens, token_seq, T, H, G, dk, dv);
+    if (taps > 1)
+      hipLaunchKernelGGL(conv_state_update_kernel<u16>, dim3(sgrid), dim3(256),
+                         0, s, conv_state, (const u16*)proj, ld, q_off, k_off,
+                         v_off, taps, state_slots, qlocs, seq_lens, S, Cq, C);
+  }
+}
+
+extern "C" void mix_delta_scan(float* o, const float* qn, const float* kn,
+                               const float* vv, const float* decay,
+                               const float* beta, float* ssm,
+                               const int* state_slots, const int* qlocs,
+                               const int* seq_lens, int S, int H, int G, int dk,
+                               int dv, hipStream_t s) {
+  int R = 1;
+  while (R * RPT < dk) R <<= 1;  // dk <= 256 -> R <= 8
+  const int cols_pb = 256 / R;
+  const int col_groups = (dv + cols_pb - 1) / cols_pb;
+  const long grid = (long)S * H * col_groups;
+  if (grid == 0) return;
+  hipLaunchKernelGGL(delta_scan_kernel, dim3((unsigned)grid), dim3(256), 0, s,
+                     o, qn, kn, vv, decay, beta, ssm, state_slots, qlocs,
+                     seq_lens, H, G, dk, dv, R, col_groups);
+}
+
+extern "C" void mix_delta_out(void* out, long ldo, int out_off, const float* o,
+                              const float* norm_w, const void* proj, long ld,
+                              int g1_off, const float* g2, int rank, float eps,
+                              float out_scale, long T, int H, int dv, int f32,
+                              hipStream_t s) {
+  const long units = T * H;
+  const int grid = (int)((units + WPB - 1) / WPB);
+  if (grid == 0) return;
+  if (f32)
+    hipLaunchKernelGGL(delta_out_kernel<float>, dim3(grid), dim3(WPB * WAVE),
+                       0, s, (float*)out, ldo, out_off, o, norm_w,
+                       (const float*)proj, ld, g1_off, g2, rank, eps,
+                       out_scale, T, H, dv);
+  else
+    hipLaunchKernelGGL(delta_out_kernel<u16>, dim3(grid), dim3(WPB * WAVE), 0,
+                       s, (u16*)out, ldo, out_off, o, norm_w,
+                       (const u16*)proj, ld, g1_off, g2, rank, eps, out_scale,
+                       T, H, dv);
+}

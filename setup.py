@@ -25,17 +25,33 @@ SOURCES = [
     "csrc/grouped_gemm.hip",
 ]
 
+# kernels of layer-list decoders (local attention, gated delta rule, gated
+# scalar-gain norms): an extension of their own, so a process that serves
+# only such a model builds and loads only these
+MIX_SOURCES = [
+    "csrc/mix_bindings.cpp",
+    "csrc/mix_norm.hip",
+    "csrc/mix_attn.hip",
+    "csrc/mix_delta.hip",
+]
+
+# hipcc's automatic packed-fp32 forms are switched off for all device code
+HIP_FLAGS = ["-O3", "--offload-arch=gfx950",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+EXTENSIONS = {"_C": SOURCES, "_C_mix": MIX_SOURCES}
+# SUTRO_AMD_EXTENSIONS=_C_mix builds only the named extensions
+_only = [n for n in os.environ.get("SUTRO_AMD_EXTENSIONS", "").split(",") if n]
+
 setup(
     name="sutro-amd-kernels",
     ext_modules=[
         CUDAExtension(
-            name="sutro_amd._C",
-            sources=SOURCES,
-            extra_compile_args={
-                "cxx": ["-O3"],
-                "nvcc": ["-O3", "--offload-arch=gfx950"],
-            },
+            name="sutro_amd." + name,
+            sources=srcs,
+            extra_compile_args={"cxx": ["-O3"], "nvcc": list(HIP_FLAGS)},
         )
+        for name, srcs in EXTENSIONS.items() if not _only or name in _only
     ],
     cmdclass={"build_ext": BuildExtension},
 )

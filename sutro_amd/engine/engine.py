@@ -303,14 +303,14 @@ class LLMEngine:
         prefill_token_count = int(qlocs[sb.num_prefills])
 
         dev = self.device
-        state_slots = token_seq = None
+        state_slots = None
         if self.kv.state is not None:
             slots_of = self.kv.state.slots
             state_slots = torch.tensor([slots_of[r.req_id] for r in sb.reqs],
                                        dtype=torch.int32, device=dev)
-            token_seq = torch.from_numpy(np.repeat(
-                np.arange(S, dtype=np.int32),
-                np.asarray(sb.num_new_tokens, dtype=np.int64))).to(dev)
+        token_seq = torch.from_numpy(np.repeat(
+            np.arange(S, dtype=np.int32),
+            np.asarray(sb.num_new_tokens, dtype=np.int64))).to(dev)
         return ForwardBatch(
             state_slots=state_slots,
             token_seq=token_seq,

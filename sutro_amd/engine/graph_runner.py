@@ -94,7 +94,7 @@ class DecodeGraphRunner:
             tile_q0=self.d_tiles,
             prefill_token_count=0,
             state_slots=self.d_state[:n] if self.has_state else None,
-            token_seq=self.d_qlocs[:n] if self.has_state else None,
+            token_seq=self.d_qlocs[:n],
         )
 
     @torch.no_grad()
@@ -194,7 +194,7 @@ class DecodeGraphRunner:
         rows = self._arange[:n]
         slots[:n] = bt[rows, p // bs].astype(np.int64) * bs + p % bs
 
-        if self.has_state:
+        if getattr(self, "has_state", False):
             st = self.h_state.numpy()
             slots_of = kv.state.slots
             st[:n] = np.fromiter((slots_of[r.req_id] for r in sb.reqs),

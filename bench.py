@@ -72,6 +72,14 @@ def build_args():
                         "its own service on its GPU (DP row shard); "
                         "standalone with --gpus N the service's own dp_pool "
                         "spawns one worker per GPU.")
+    p.add_argument("--arch-compare", type=str, default=None, metavar="SIZES",
+                   help="instead of the flagship workload: prefill and decode "
+                        "tokens/s of the Vodinex layer-list decoder beside "
+                        "the Qwen3 dense decoder of equal size, random "
+                        "weights (comma list of 1b,8b,tiny); one JSON line "
+                        "per model")
+    p.add_argument("--compare-seqs", type=int, default=16)
+    p.add_argument("--compare-prompt", type=int, default=2048)
     p.add_argument("--e2e-rows", type=int, default=3000,
                    help="rows per GPU for --e2e")
     return p.parse_args()
@@ -240,6 +248,17 @@ def main():
         dist = dist_mod
         backend = "nccl" if have_gpu else "gloo"
         dist.init_process_group(backend=backend)
+
+    if args.arch_compare:
+        from sutro_amd.utils.arch_bench import run_compare
+
+        rows = run_compare(args.arch_compare.split(","), device,
+                           args.compare_seqs, args.compare_prompt,
+                           steps=args.steps, warmup=args.warmup)
+        if rank == 0:
+            for r in rows:
+                print(json.dumps(r))
+        return
 
     if args.e2e:
         run_e2e(args, rank, world, local_rank, have_gpu)

@@ -86,16 +86,16 @@ __global__ void local_attention_kernel(
     const int* __restrict__ bt, int bt_stride, const int* __restrict__ seq_lens,
     const int* __restrict__ qlocs, const int* __restrict__ token_seq,
     float scale, int chunk, int window, const A* __restrict__ proj, long ld,
-    int gate_off, float out_scale, long T, int H, int G, int dk, int dv,
-    int page) {
+    int gate_off, float out_scale, long t0, long T, int H, int G, int dk,
+    int dv, int page) {
   extern __shared__ float sm[];  // WPB * dk floats: the wave's query
   const int lane = threadIdx.x & (WAVE - 1);
   const int wid = threadIdx.x / WAVE;
   float* qs = sm + wid * dk;
   const long u = (long)blockIdx.x * WPB + wid;
   const bool valid = u < T * H;
-  const long t = valid ? u / H : 0;
-  const int h = valid ? (int)(u - t * H) : 0;
+  const long t = t0 + (valid ? u / H : 0);  // rows [t0, t0 + T)
+  const int h = valid ? (int)(u % H) : 0;
   const int g = h / (H / G);
   for (int i = lane; i < dk; i += WAVE)
     qs[i] = ldf<A>(q + (t * H + h) * (long)dk + i);
@@ -188,7 +188,7 @@ static void launch_local_attention(
     const void* v_cache, const int* bt, int bt_stride, const int* seq_lens,
     const int* qlocs, const int* token_seq, float scale, int chunk,
     int window, const void* proj, long ld, int gate_off, float out_scale,
-    long T, int H, int G, int dk, int dv, int page, hipStream_t s) {
+    long t0, long T, int H, int G, int dk, int dv, int page, hipStream_t s) {
   const long units = T * H;
   const int grid = (int)((units + WPB - 1) / WPB);
   if (grid == 0) return;
@@ -198,8 +198,8 @@ static void launch_local_attention(
                      dim3(WPB * WAVE), smem, s, (A*)out, ldo, out_off,       \
                      (const A*)q, (const A*)k_cache, (const A*)v_cache, bt,  \
                      bt_stride, seq_lens, qlocs, token_seq, scale, chunk,    \
-                     window, (const A*)proj, ld, gate_off, out_scale, T, H,  \
-                     G, dk, dv, page)
+                     window, (const A*)proj, ld, gate_off, out_scale, t0, T, \
+                     H, G, dk, dv, page)
   if (dv <= 64) LAUNCH_LA(1);
   else if (dv <= 128) LAUNCH_LA(2);
   else LAUNCH_LA(4);
@@ -211,15 +211,16 @@ extern "C" void mix_local_attention(
     const void* v_cache, const int* bt, int bt_stride, const int* seq_lens,
     const int* qlocs, const int* token_seq, float scale, int chunk,
     int window, const void* proj, long ld, int gate_off, float out_scale,
-    long T, int H, int G, int dk, int dv, int page, int f32, hipStream_t s) {
+    long t0, long T, int H, int G, int dk, int dv, int page, int f32,
+    hipStream_t s) {
   if (f32)
     launch_local_attention<float>(out, ldo, out_off, q, k_cache, v_cache, bt,
                                   bt_stride, seq_lens, qlocs, token_seq, scale,
                                   chunk, window, proj, ld, gate_off, out_scale,
-                                  T, H, G, dk, dv, page, s);
+                                  t0, T, H, G, dk, dv, page, s);
   else
     launch_local_attention<u16>(out, ldo, out_off, q, k_cache, v_cache, bt,
                                 bt_stride, seq_lens, qlocs, token_seq, scale,
                                 chunk, window, proj, ld, gate_off, out_scale,
-                                T, H, G, dk, dv, page, s);
+                                t0, T, H, G, dk, dv, page, s);
 }

@@ -50,8 +50,13 @@ void mix_attn_prep(void*, const void*, long, int, int, int, const float*,
 void mix_local_attention(void*, long, int, const void*, const void*,
                          const void*, const int*, int, const int*, const int*,
                          const int*, float, int, int, const void*, long, int,
-                         float, long, int, int, int, int, int, int,
+                         float, long, long, int, int, int, int, int, int,
                          hipStream_t);
+int mix_local_attention_mfma(void*, long, int, const void*, const void*,
+                             const void*, const int*, int, const int*,
+                             const int*, const int*, const int*, int, float,
+                             int, int, const void*, long, int, float, int, int,
+                             int, int, int, hipStream_t);
 void mix_delta_prep(float*, float*, float*, float*, float*, const void*, long,
                     int, int, int, int, int, const float*, int, const float*,
                     int, const float*, const float*, float*, const int*,
@@ -160,7 +165,10 @@ void local_attention(torch::Tensor out, long out_off, torch::Tensor q,
                      torch::Tensor bt, torch::Tensor seq_lens,
                      torch::Tensor qlocs, torch::Tensor token_seq,
                      double scale, long chunk, long window, torch::Tensor proj,
-                     long gate_off, double out_scale) {
+                     long gate_off, double out_scale,
+                     c10::optional<torch::Tensor> tile_seq,
+                     c10::optional<torch::Tensor> tile_q0,
+                     long prefill_rows) {
   CHECK_GPU(q); CHECK_CONTIG(q); CHECK_CONTIG(k_cache); CHECK_CONTIG(v_cache);
   CHECK_I32(bt); CHECK_I32(seq_lens); CHECK_I32(qlocs); CHECK_I32(token_seq);
   CHECK_CONTIG(bt);
@@ -180,14 +188,35 @@ void local_attention(torch::Tensor out, long out_off, torch::Tensor q,
               bt.size(0) == seq_lens.numel(), "batch metadata sizes");
   if (gate_off >= 0) check_proj(proj, gate_off, H, "gate");
   TORCH_CHECK(proj.size(0) == T, "row mismatch");
-  mix_local_attention(out.data_ptr(), out.stride(0), (int)out_off,
-                      q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
-                      bt.data_ptr<int>(), (int)bt.size(1),
-                      seq_lens.data_ptr<int>(), qlocs.data_ptr<int>(),
-                      token_seq.data_ptr<int>(), (float)scale, (int)chunk,
-                      (int)window, proj.data_ptr(), proj.stride(0),
-                      (int)gate_off, (float)out_scale, T, (int)H, (int)G,
-                      (int)dk, (int)dv, (int)page, act_kind(q), cur_stream());
+  // prompt pieces (the first `prefill_rows` rows, tiled 32 rows a tile by
+  // tile_seq / tile_q0) go to the MFMA kernel when the shape allows it;
+  // single-token rows and every other shape go to the generic kernel
+  long t0 = 0;
+  if (act_kind(q) == 0 && tile_seq.has_value() && tile_q0.has_value() &&
+      prefill_rows > 0) {
+    CHECK_I32(*tile_seq); CHECK_I32(*tile_q0);
+    TORCH_CHECK(tile_seq->numel() == tile_q0->numel() && prefill_rows <= T,
+                "tile map sizes");
+    if (mix_local_attention_mfma(
+            out.data_ptr(), out.stride(0), (int)out_off, q.data_ptr(),
+            k_cache.data_ptr(), v_cache.data_ptr(), bt.data_ptr<int>(),
+            (int)bt.size(1), seq_lens.data_ptr<int>(), qlocs.data_ptr<int>(),
+            tile_seq->data_ptr<int>(), tile_q0->data_ptr<int>(),
+            (int)tile_seq->numel(), (float)scale, (int)chunk, (int)window,
+            proj.data_ptr(), proj.stride(0), (int)gate_off, (float)out_scale,
+            (int)H, (int)G, (int)dk, (int)dv, (int)page, cur_stream()))
+      t0 = prefill_rows;
+  }
+  if (t0 < T)
+    mix_local_attention(out.data_ptr(), out.stride(0), (int)out_off,
+                        q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                        bt.data_ptr<int>(), (int)bt.size(1),
+                        seq_lens.data_ptr<int>(), qlocs.data_ptr<int>(),
+                        token_seq.data_ptr<int>(), (float)scale, (int)chunk,
+                        (int)window, proj.data_ptr(), proj.stride(0),
+                        (int)gate_off, (float)out_scale, t0, T - t0, (int)H,
+                        (int)G, (int)dk, (int)dv, (int)page, act_kind(q),
+                        cur_stream());
 }
 
 void delta_prep(torch::Tensor qn, torch::Tensor kn, torch::Tensor v,
@@ -210,11 +239,11 @@ void delta_prep(torch::Tensor qn, torch::Tensor kn, torch::Tensor v,
   const long G = qn.size(1), dk = qn.size(2);
   const long S = seq_lens.numel();
   const long C = 2 * G * dk + H * dv, taps = conv_w.size(1);
-  const long rank = a2.size(1);
+  const long rank = a2.size(0);  // a2 arrives transposed: [rank, H*dk]
   TORCH_CHECK(dk <= 256 && dv <= 256, "head sizes above 256 are unsupported");
   TORCH_CHECK(H % G == 0, "heads must be a multiple of kv heads");
   TORCH_CHECK(conv_w.size(0) == C, "filter channels");
-  TORCH_CHECK(a2.size(0) == H * dk && dt_bias.numel() == H * dk &&
+  TORCH_CHECK(a2.size(1) == H * dk && dt_bias.numel() == H * dk &&
               a_log.numel() == H, "decay parameter sizes");
   TORCH_CHECK(conv_state.dim() == 3 && conv_state.size(2) == C &&
               conv_state.size(1) >= taps - 1 &&
@@ -275,8 +304,8 @@ void delta_out(torch::Tensor out, long out_off, torch::Tensor o,
   CHECK_GPU(o); CHECK_F32(o); CHECK_CONTIG(o); CHECK_F32(norm_w);
   CHECK_F32(g2); CHECK_CONTIG(g2);
   const long T = o.size(0), H = o.size(1), dv = o.size(2);
-  const long rank = g2.size(1);
-  TORCH_CHECK(norm_w.numel() == dv && g2.size(0) == H * dv, "parameter sizes");
+  const long rank = g2.size(0);  // g2 arrives transposed: [rank, H*dv]
+  TORCH_CHECK(norm_w.numel() == dv && g2.size(1) == H * dv, "parameter sizes");
   TORCH_CHECK(out.dim() == 2 && out.stride(1) == 1 && out.size(0) == T &&
               out_off >= 0 && out_off + H * dv <= out.size(1), "out section");
   TORCH_CHECK(out.scalar_type() == proj.scalar_type(), "dtype mismatch");
@@ -296,7 +325,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("scalar_rmsnorm", &scalar_rmsnorm, "RMS norm with one scalar gain");
   m.def("attn_prep", &attn_prep, "q/k norm + partial rotation + paged K/V write");
   m.def("local_attention", &local_attention,
-        "chunked/windowed paged attention with per-head output gate");
+        "chunked/windowed paged attention with per-head output gate",
+        py::arg("out"), py::arg("out_off"), py::arg("q"), py::arg("k_cache"),
+        py::arg("v_cache"), py::arg("bt"), py::arg("seq_lens"),
+        py::arg("qlocs"), py::arg("token_seq"), py::arg("scale"),
+        py::arg("chunk"), py::arg("window"), py::arg("proj"),
+        py::arg("gate_off"), py::arg("out_scale"),
+        py::arg("tile_seq") = c10::nullopt, py::arg("tile_q0") = c10::nullopt,
+        py::arg("prefill_rows") = 0);
   m.def("delta_prep", &delta_prep, "delta-rule inputs: filters, norms, gates");
   m.def("delta_scan", &delta_scan, "gated delta rule over new tokens");
   m.def("delta_out", &delta_out, "per-head norm + low-rank gate of the read-out");

@@ -51,10 +51,12 @@ __global__ void delta_prep_kernel(
     const int h = j - 2 * G - H;
     const A* a1 = proj + t * ld + a1_off;
     const float rate = expf(a_log[h]);
+    const long HD = (long)H * dk;
     for (int i = lane; i < dk; i += WAVE) {
-      const float* w = a2 + ((long)h * dk + i) * rank;
+      // a2 is stored transposed [rank, H*dk]: lanes read consecutive floats
+      const float* w = a2 + (long)h * dk + i;
       float a = dt_bias[h * dk + i];
-      for (int r = 0; r < rank; ++r) a += w[r] * ldf<A>(a1 + r);
+      for (int r = 0; r < rank; ++r) a += w[r * HD] * ldf<A>(a1 + r);
       decay[(t * H + h) * (long)dk + i] = expf(-rate * softplus_f(a));
     }
     if (lane == 0)
@@ -213,10 +215,12 @@ __global__ void delta_out_kernel(A* __restrict__ out, long ldo, int out_off,
   ssq = wave_sum_f32(ssq);
   const float inv = out_scale / sqrtf(ssq / (float)dv + eps);
   const A* g1 = proj + t * ld + g1_off;
+  const long HV = (long)H * dv;
   for (int c = lane; c < dv; c += WAVE) {
-    const float* w = g2 + ((long)h * dv + c) * rank;
+    // g2 is stored transposed [rank, H*dv]
+    const float* w = g2 + (long)h * dv + c;
     float a = 0.f;
-    for (int r = 0; r < rank; ++r) a += w[r] * ldf<A>(g1 + r);
+    for (int r = 0; r < rank; ++r) a += w[r * HV] * ldf<A>(g1 + r);
     stf<A>(out + t * ldo + out_off + (long)h * dv + c,
            orow[c] * inv * norm_w[c] * sigmoid_f(a));
   }

@@ -32,6 +32,7 @@ MIX_SOURCES = [
     "csrc/mix_bindings.cpp",
     "csrc/mix_norm.hip",
     "csrc/mix_attn.hip",
+    "csrc/mix_attn_mfma.hip",
     "csrc/mix_delta.hip",
 ]
 

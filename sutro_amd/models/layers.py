@@ -121,7 +121,8 @@ class LocalAttention(nn.Module):
             q, kc, vc, fb.block_tables, fb.seq_lens, fb.query_start_locs,
             s.scale, s.chunk, s.window, proj,
             off[tag + "g"] if s.out_gate else -1, out, out_off, out_scale,
-            token_seq=fb.token_seq, max_query_len=fb.max_query_len)
+            token_seq=fb.token_seq, tile_seq=fb.tile_seq, tile_q0=fb.tile_q0,
+            prefill_rows=fb.prefill_token_count)
 
 
 class GatedDeltaRule(nn.Module):
@@ -150,6 +151,7 @@ class GatedDeltaRule(nn.Module):
         self.norm_w = nn.Parameter(torch.ones(spec.vdim, dtype=f32))
         self.g2 = nn.Parameter(torch.zeros(spec.heads * spec.vdim,
                                            spec.gate_rank, dtype=f32))
+        self._t = None
 
     def in_sections(self, tag: str):
         s = self.spec
@@ -189,13 +191,18 @@ class GatedDeltaRule(nn.Module):
                 out_off: int, out_scale: float) -> None:
         s = self.spec
         st = kv.state
+        if self._t is None or self._t[0].device != proj.device:
+            # transposed copies of the low-rank up-projections, made once
+            # (before any graph capture: capture is preceded by a warm-up run)
+            self._t = (self.a2.detach().t().contiguous(),
+                       self.g2.detach().t().contiguous())
         qn, kn, v, decay, beta = hops.delta_prep(
             proj, off[tag + "q"], off[tag + "k"], off[tag + "v"],
             off[tag + "b"], off[tag + "a1"], s.heads, s.kv_heads, s.dim,
             s.vdim, self.conv_w, self.a2, self.dt_bias, self.a_log,
             st.conv[self.layer_idx], fb.state_slots, fb.query_start_locs,
-            fb.seq_lens, token_seq=fb.token_seq)
+            fb.seq_lens, token_seq=fb.token_seq, a2_t=self._t[0])
         o = hops.delta_scan(qn, kn, v, decay, beta, st.ssm[self.layer_idx],
                             fb.state_slots, fb.query_start_locs, fb.seq_lens)
         hops.delta_out(o, self.norm_w, proj, off[tag + "g1"], self.g2,
-                       self.eps, out, out_off, out_scale)
+                       self.eps, out, out_off, out_scale, g2_t=self._t[1])

@@ -84,12 +84,21 @@ def attn_prep(proj, q_off, k_off, v_off, H, G, dk, dv, q_norm_w, k_norm_w,
 def local_attention(q, k_cache, v_cache, block_tables, seq_lens,
                     query_start_locs, scale: float, chunk: int, window: int,
                     proj, gate_off: int, out, out_off: int, out_scale: float,
-                    token_seq=None, max_query_len: int = 0):
+                    token_seq=None, tile_seq=None, tile_q0=None,
+                    prefill_rows: int = 0):
+    """`tile_seq`/`tile_q0` (int32, 32 query rows a tile) cover the first
+    `prefill_rows` rows: on the GPU in bf16 those rows run on the MFMA kernel
+    when page size and head sizes allow it; the remaining (single-token) rows
+    and all other cases run on the generic one-wave-per-row kernel."""
     if q.is_cuda:
+        if tile_seq is None or tile_seq.numel() == 0:
+            tile_seq = tile_q0 = None
+            prefill_rows = 0
         _mix().local_attention(out, out_off, q, k_cache, v_cache,
                                block_tables, seq_lens, query_start_locs,
                                token_seq, scale, chunk, window, proj,
-                               gate_off, out_scale)
+                               gate_off, out_scale, tile_seq, tile_q0,
+                               prefill_rows)
         return
     torch_ref.local_attention(q, k_cache, v_cache, block_tables, seq_lens,
                               query_start_locs, scale, chunk, window, proj,
@@ -98,8 +107,12 @@ def local_attention(q, k_cache, v_cache, block_tables, seq_lens,
 
 def delta_prep(proj, q_off, k_off, v_off, b_off, a1_off, H, G, dk, dv,
                conv_w, a2, dt_bias, a_log, conv_state, state_slots,
-               query_start_locs, seq_lens, token_seq=None):
+               query_start_locs, seq_lens, token_seq=None, a2_t=None):
+    """`a2_t`: a2 transposed and contiguous ([rank, H*dk], what the kernel
+    reads); made on the fly when the caller does not keep one."""
     if proj.is_cuda:
+        if a2_t is None:
+            a2_t = a2.t().contiguous()
         T = proj.shape[0]
         f32 = dict(dtype=torch.float32, device=proj.device)
         qn = torch.empty((T, G, dk), **f32)
@@ -108,7 +121,7 @@ def delta_prep(proj, q_off, k_off, v_off, b_off, a1_off, H, G, dk, dv,
         decay = torch.empty((T, H, dk), **f32)
         beta = torch.empty((T, H), **f32)
         _mix().delta_prep(qn, kn, v, decay, beta, proj, q_off, k_off, v_off,
-                          b_off, a1_off, conv_w, a2, dt_bias, a_log,
+                          b_off, a1_off, conv_w, a2_t, dt_bias, a_log,
                           conv_state, state_slots, query_start_locs, seq_lens,
                           token_seq)
         return qn, kn, v, decay, beta
@@ -130,9 +143,11 @@ def delta_scan(qn, kn, v, decay, beta, ssm_state, state_slots,
 
 
 def delta_out(o, norm_w, proj, g1_off: int, g2, eps: float, out,
-              out_off: int, out_scale: float) -> None:
+              out_off: int, out_scale: float, g2_t=None) -> None:
     if o.is_cuda:
-        _mix().delta_out(out, out_off, o, norm_w, proj, g1_off, g2, eps,
+        if g2_t is None:
+            g2_t = g2.t().contiguous()
+        _mix().delta_out(out, out_off, o, norm_w, proj, g1_off, g2_t, eps,
                          out_scale)
         return
     torch_ref.delta_out(o, norm_w, proj, g1_off, g2, eps, out, out_off,

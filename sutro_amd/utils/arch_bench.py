@@ -1,0 +1,124 @@
+"""Prefill and decode throughput of a layer-list decoder beside the Qwen3
+dense decoder of equal size (same width, layers, heads, key/value heads, head
+size and feed-forward width), both with random weights, both through the
+engine's own batch path (scheduler, paged cache, state slots, decode
+hipGraphs). Used by `bench.py --arch-compare`.
+
+prefill: `seqs` prompts of `prompt` tokens in one engine step, tokens/s.
+decode:  `seqs` sequences, each with `prompt` tokens of context, one token a
+         step through the captured decode graph, tokens/s.
+"""
+
+from __future__ import annotations
+
+import time
+from typing import Dict, List
+
+import torch
+
+from ..engine.config import EngineConfig
+from ..engine.engine import LLMEngine
+from ..models.hybrid_spec import (AttnMixerSpec, DeltaMixerSpec,
+                                  HybridLayerSpec, HybridSpec,
+                                  ParallelMixerSpec)
+from ..models.registry import ModelSpec
+
+# name -> (width, layers, heads, kv_heads, head size, ff, vocab)
+SIZES = {
+    "1b": (2048, 4, 16, 4, 128, 8192, 32768),
+    "8b": (4096, 4, 32, 8, 128, 12288, 32768),
+    "tiny": (192, 2, 3, 1, 64, 384, 320),
+}
+
+
+def hybrid_spec(name: str, chunk: int = 1024) -> HybridSpec:
+    W, L, H, G, D, ff, V = SIZES[name]
+    left = AttnMixerSpec(heads=H, kv_heads=G, dim=D, vdim=D, scale=D ** -0.5,
+                         rot_dims=D // 2, rot_base=10000.0, chunk=chunk)
+    right = DeltaMixerSpec(heads=H // 2, kv_heads=H // 2, dim=D, vdim=D, conv=4,
+                           decay_rank=32, gate_rank=32)
+    solo = DeltaMixerSpec(heads=H, kv_heads=H, dim=D, vdim=D, conv=4,
+                          decay_rank=32, gate_rank=32)
+    layers: List[HybridLayerSpec] = []
+    for i in range(L):
+        if i == 0:
+            layers.append(HybridLayerSpec("channel_delta", solo, ff=ff))
+        else:
+            layers.append(HybridLayerSpec(
+                "parallel", ParallelMixerSpec(left, right, 0.75, 0.4), ff=ff))
+    return HybridSpec(name=f"vodinex-{name}", arch="vodinex", hidden_size=W,
+                      vocab_size=V, layers=tuple(layers), norm_eps=1e-6,
+                      residual_mult=0.8, max_context=1 << 20)
+
+
+def dense_spec(name: str) -> ModelSpec:
+    W, L, H, G, D, ff, V = SIZES[name]
+    return ModelSpec(name=f"qwen3-{name}", arch="qwen3", hidden_size=W,
+                     num_layers=L, num_heads=H, num_kv_heads=G, head_dim=D,
+                     intermediate_size=ff, vocab_size=V, max_context=1 << 20)
+
+
+def _measure(spec, device: str, seqs: int, prompt: int, steps: int,
+             warmup: int) -> Dict[str, float]:
+    page = 32
+    blocks = seqs * ((prompt + steps + warmup + 2 * page) // page + 1) + 2
+    cfg = EngineConfig(spec=spec, device=device, max_model_len=prompt + steps
+                       + warmup + 2 * page, max_num_seqs=seqs,
+                       num_kv_blocks=blocks,
+                       max_tokens_per_step=seqs * prompt + seqs)
+    eng = LLMEngine(cfg)
+    g = torch.Generator().manual_seed(0)
+
+    def sync():
+        if device.startswith("cuda"):
+            torch.cuda.synchronize()
+
+    def prompts():
+        return [torch.randint(3, spec.vocab_size, (prompt,), generator=g).tolist()
+                for _ in range(seqs)]
+
+    def prefill():
+        reqs = [eng.new_replay_request() for _ in range(seqs)]
+        toks = prompts()
+        sync()
+        t0 = time.perf_counter()
+        eng.replay_step([(r, t, [prompt - 1]) for r, t in zip(reqs, toks)])
+        sync()
+        return reqs, time.perf_counter() - t0
+
+    # prefill: first pass warms GEMM selection, later ones are timed
+    times = []
+    reqs = None
+    for i in range(3):
+        if reqs is not None:
+            for r in reqs:
+                eng.finish_replay_request(r)
+        reqs, dt = prefill()
+        if i:
+            times.append(dt)
+    out = {"prefill_tok_s": seqs * prompt / min(times)}
+    # decode: continue the last prefilled batch
+    for i in range(warmup + steps):
+        if i == warmup:
+            sync()
+            t0 = time.perf_counter()
+        eng.replay_step([(r, [7 + i % 11], [0]) for r in reqs])
+    sync()
+    out["decode_tok_s"] = seqs * steps / (time.perf_counter() - t0)
+    out["decode_graph"] = eng.graph_runner is not None
+    return out
+
+
+def run_compare(sizes: List[str], device: str, seqs: int, prompt: int,
+                steps: int, warmup: int) -> List[dict]:
+    rows = []
+    for name in sizes:
+        for kind, spec in (("vodinex", hybrid_spec(name)),
+                           ("qwen3", dense_spec(name))):
+            r = _measure(spec, device, seqs, prompt, steps, warmup)
+            r.update(model=spec.name, kind=kind, size=name, seqs=seqs,
+                     prompt=prompt, params=spec.param_count())
+            rows.append(r)
+            if device.startswith("cuda"):
+                torch.cuda.empty_cache()
+    return rows

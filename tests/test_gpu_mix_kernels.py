@@ -59,6 +59,7 @@ def _batch(lens_new, lens_total, page, n_blocks, seed):
     S = len(lens_new)
     perm = torch.randperm(n_blocks - 1, generator=g) + 1
     per = (n_blocks - 1) // S          # every sequence draws from its own run
+    per = max(per, 1)
     tables = []
     for s, L in enumerate(lens_total):
         nb = (L + page - 1) // page
@@ -209,3 +210,55 @@ def test_delta_rule_ops(dtype, H, G, dk, dv, taps, rank):
         hops.delta_out(o_r.to(DEV), norm_w.to(DEV), proj.to(DEV), g1_off,
                        g2.to(DEV), 2e-5, out_d, 16, 0.45)
         _close(out_d, out_r, dtype)
+
+
+@pytest.mark.parametrize("H,G,dk,dv,chunk,window", [
+    (4, 2, 64, 56, 48, 0),
+    (8, 2, 128, 128, 100, 0),
+    (6, 3, 40, 72, 0, 45),
+    (2, 1, 256, 136, 37, 50),
+    (16, 1, 64, 64, 0, 0),
+])
+def test_local_attention_matrix_core_path(H, G, dk, dv, chunk, window):
+    """bf16, page 32: prompt pieces run on the MFMA kernel (tile map given),
+    trailing single-token rows on the generic kernel; both against the fp32
+    reference. Pieces start inside pages and inside chunks."""
+    dtype = torch.bfloat16
+    page, n_blocks = 32, 41
+    g = torch.Generator().manual_seed(13)
+    kc = torch.zeros(n_blocks, G, page, dk, dtype=dtype)
+    vc = torch.zeros(n_blocks, G, page, dv, dtype=dtype)
+    inv = ref.rope_inv_freq(0, 1.0)
+    q_off, k_off = 0, H * dk
+    v_off = k_off + G * dk
+    g_off = v_off + _round8(G * dv)
+    ncol = g_off + _round8(H)
+    steps = [([150, 33, 5, 70], [150, 33, 5, 70], 4),
+             ([61, 40, 1, 1], [211, 73, 6, 71], 2),
+             ([95, 1, 1, 1], [306, 74, 7, 72], 1)]
+    for lens_new, lens_total, n_prefill in steps:
+        b = _batch(lens_new, lens_total, page, n_blocks, 5)
+        T = sum(lens_new)
+        proj = torch.randn(T, ncol, generator=g).to(dtype)
+        qr = ref.attn_prep(proj, q_off, k_off, v_off, H, G, dk, dv, None, None,
+                           2e-5, inv, b["pos"], b["slots"], kc, vc)
+        out_r = torch.zeros(T, H * dv, dtype=torch.float32)
+        ref.local_attention(qr.float(), kc.float(), vc.float(), b["bt"],
+                            b["seq_lens"], b["qlocs"], dk ** -0.5, chunk,
+                            window, proj, g_off, out_r, 0, 0.55)
+        tiles_s, tiles_q0 = [], []
+        for s in range(n_prefill):
+            for j in range(0, lens_new[s], 32):
+                tiles_s.append(s)
+                tiles_q0.append(j)
+        out_d = torch.zeros(T, H * dv, dtype=dtype, device=DEV)
+        hops.local_attention(
+            qr.to(DEV), kc.to(DEV), vc.to(DEV), b["bt"].to(DEV),
+            b["seq_lens"].to(DEV), b["qlocs"].to(DEV), dk ** -0.5, chunk,
+            window, proj.to(DEV), g_off, out_d, 0, 0.55,
+            token_seq=b["token_seq"].to(DEV),
+            tile_seq=torch.tensor(tiles_s, dtype=torch.int32, device=DEV),
+            tile_q0=torch.tensor(tiles_q0, dtype=torch.int32, device=DEV),
+            prefill_rows=sum(lens_new[:n_prefill]))
+        torch.testing.assert_close(out_d.float().cpu(), out_r, rtol=2e-2,
+                                   atol=2e-2)

@@ -134,65 +134,137 @@ __global__ void conv_state_update_kernel(
 }
 
 #define RPT 32  // state rows per lane
+#define TB 8    // tokens staged per step
 
-__global__ void delta_scan_kernel(
+// Token-by-token scan. Block = (sequence, head, group of 256/R columns);
+// lane (col, r) keeps rows {((n/4)*R + r)*4 + n%4 : n < 32} of its column of
+// S in registers (rows past dk stay zero: their k and q are staged as 0 and
+// their decay as 1). k, q, decay, v and beta of TB tokens at a time are
+// staged through a double-buffered LDS tile: the global loads of tile s+1
+// are issued before the arithmetic of tile s and parked in registers. With
+// this row mapping the R lanes of a column read consecutive float4s of a
+// staged row, and all columns read the same addresses (LDS broadcast).
+template <int R>
+__global__ void __launch_bounds__(256) delta_scan_kernel(
     float* __restrict__ o, const float* __restrict__ qn,
     const float* __restrict__ kn, const float* __restrict__ vv,
     const float* __restrict__ decay, const float* __restrict__ beta,
     float* __restrict__ ssm, const int* __restrict__ state_slots,
     const int* __restrict__ qlocs, const int* __restrict__ seq_lens, int H,
-    int G, int dk, int dv, int R, int col_groups) {
-  const int cols_pb = blockDim.x / R;
+    int G, int dk, int dv, int col_groups) {
+  constexpr int DKP = R * RPT;
+  constexpr int CPB = 256 / R;            // columns per block
+  constexpr int NK = 3 * TB * DKP / 256;  // staged k|q|decay floats per lane
+  constexpr int NV = TB * CPB / 256 > 0 ? TB * CPB / 256 : 1;
+  constexpr int TILE = 3 * TB * DKP + TB * CPB + TB;
+  __shared__ __attribute__((aligned(16))) float lds[2][TILE];
+
   int b = blockIdx.x;
   const int cg = b % col_groups; b /= col_groups;
   const int h = b % H;
   const int s = b / H;
-  const int r = threadIdx.x % R;
-  const int col = cg * cols_pb + threadIdx.x / R;
+  const int tid = threadIdx.x;
+  const int r = tid % R;
+  const int cl = tid / R;                 // column within the block
+  const int col = cg * CPB + cl;
   const bool cv = col < dv;
   const int g = h / (H / G);
   const int q0 = qlocs[s], q1 = qlocs[s + 1];
   if (q1 <= q0) return;
   const int start = seq_lens[s] - (q1 - q0);
-  const int i0 = r * RPT;
   float* Sg = ssm + (((long)state_slots[s] * H + h) * dk) * dv;
 
   float S[RPT];
 #pragma unroll
-  for (int i = 0; i < RPT; ++i)
-    S[i] = (start > 0 && cv && i0 + i < dk) ? Sg[(long)(i0 + i) * dv + col]
-                                            : 0.f;
+  for (int n = 0; n < RPT; ++n) {
+    const int i = ((n >> 2) * R + r) * 4 + (n & 3);
+    S[n] = (start > 0 && cv && i < dk) ? Sg[(long)i * dv + col] : 0.f;
+  }
 
-  for (int t = q0; t < q1; ++t) {
-    const float* kt = kn + ((long)t * G + g) * dk + i0;
-    const float* qt = qn + ((long)t * G + g) * dk + i0;
-    const float* dt = decay + ((long)t * H + h) * dk + i0;
-    const float vt = cv ? vv[((long)t * H + h) * dv + col] : 0.f;
-    const float bt = beta[(long)t * H + h];
-    float kk[RPT];
-    float dot = 0.f;
+  float pk[NK], pv[NV], pb = 0.f;
+  auto prefetch = [&](int t0) {
 #pragma unroll
-    for (int i = 0; i < RPT; ++i) {
-      const bool in = i0 + i < dk;
-      kk[i] = in ? kt[i] : 0.f;
-      S[i] *= in ? dt[i] : 1.f;
-      dot += S[i] * kk[i];
+    for (int n = 0; n < NK; ++n) {
+      const int e = tid + n * 256;
+      const int arr = e / (TB * DKP), rem = e % (TB * DKP);
+      const int tok = rem / DKP, i = rem % DKP;
+      const int t = t0 + tok;
+      float x = arr == 2 ? 1.f : 0.f;
+      if (t < q1 && i < dk) {
+        if (arr == 0) x = kn[((long)t * G + g) * dk + i];
+        else if (arr == 1) x = qn[((long)t * G + g) * dk + i];
+        else x = decay[((long)t * H + h) * dk + i];
+      }
+      pk[n] = x;
     }
-    for (int off = R >> 1; off > 0; off >>= 1) dot += __shfl_xor(dot, off, WAVE);
-    const float uu = bt * (vt - dot);
-    float out = 0.f;
 #pragma unroll
-    for (int i = 0; i < RPT; ++i) {
-      S[i] += kk[i] * uu;
-      out += S[i] * (i0 + i < dk ? qt[i] : 0.f);
+    for (int n = 0; n < NV; ++n) {
+      const int e = tid + n * 256;
+      const int tok = e / CPB, c = cg * CPB + e % CPB;
+      const int t = t0 + tok;
+      pv[n] = (e < TB * CPB && t < q1 && c < dv)
+                  ? vv[((long)t * H + h) * dv + c] : 0.f;
     }
-    for (int off = R >> 1; off > 0; off >>= 1) out += __shfl_xor(out, off, WAVE);
-    if (r == 0 && cv) o[((long)t * H + h) * dv + col] = out;
+    if (tid < TB) pb = t0 + tid < q1 ? beta[(long)(t0 + tid) * H + h] : 0.f;
+  };
+
+  prefetch(q0);
+  int buf = 0;
+  for (int t0 = q0; t0 < q1; t0 += TB, buf ^= 1) {
+    float* L = lds[buf];
+#pragma unroll
+    for (int n = 0; n < NK; ++n) L[tid + n * 256] = pk[n];
+#pragma unroll
+    for (int n = 0; n < NV; ++n)
+      if (tid + n * 256 < TB * CPB) L[3 * TB * DKP + tid + n * 256] = pv[n];
+    if (tid < TB) L[3 * TB * DKP + TB * CPB + tid] = pb;
+    __syncthreads();
+    if (t0 + TB < q1) prefetch(t0 + TB);
+    const int nt = min(TB, q1 - t0);
+    for (int tok = 0; tok < nt; ++tok) {
+      const f32x4* K4 = (const f32x4*)(L + tok * DKP);
+      const f32x4* Q4 = (const f32x4*)(L + (TB + tok) * DKP);
+      const f32x4* D4 = (const f32x4*)(L + (2 * TB + tok) * DKP);
+      const float vt = L[3 * TB * DKP + tok * CPB + cl];
+      const float bt = L[3 * TB * DKP + TB * CPB + tok];
+      float kk[RPT];
+      float dot = 0.f;
+#pragma unroll
+      for (int m = 0; m < RPT / 4; ++m) {
+        const f32x4 k4 = K4[m * R + r], d4 = D4[m * R + r];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          kk[m * 4 + j] = k4[j];
+          S[m * 4 + j] *= d4[j];
+          dot += S[m * 4 + j] * k4[j];
+        }
+      }
+#pragma unroll
+      for (int off = R >> 1; off > 0; off >>= 1)
+        dot += __shfl_xor(dot, off, WAVE);
+      const float uu = bt * (vt - dot);
+      float out = 0.f;
+#pragma unroll
+      for (int m = 0; m < RPT / 4; ++m) {
+        const f32x4 q4 = Q4[m * R + r];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          S[m * 4 + j] += kk[m * 4 + j] * uu;
+          out += S[m * 4 + j] * q4[j];
+        }
+      }
+#pragma unroll
+      for (int off = R >> 1; off > 0; off >>= 1)
+        out += __shfl_xor(out, off, WAVE);
+      if (r == 0 && cv) o[((long)(t0 + tok) * H + h) * dv + col] = out;
+    }
   }
   if (cv) {
 #pragma unroll
-    for (int i = 0; i < RPT; ++i)
-      if (i0 + i < dk) Sg[(long)(i0 + i) * dv + col] = S[i];
+    for (int n = 0; n < RPT; ++n) {
+      const int i = ((n >> 2) * R + r) * 4 + (n & 3);
+      if (i < dk) Sg[(long)i * dv + col] = S[n];
+    }
   }
 }
 
@@ -276,9 +348,15 @@ extern "C" void mix_delta_scan(float* o, const float* qn, const float* kn,
   const int col_groups = (dv + cols_pb - 1) / cols_pb;
   const long grid = (long)S * H * col_groups;
   if (grid == 0) return;
-  hipLaunchKernelGGL(delta_scan_kernel, dim3((unsigned)grid), dim3(256), 0, s,
-                     o, qn, kn, vv, decay, beta, ssm, state_slots, qlocs,
-                     seq_lens, H, G, dk, dv, R, col_groups);
+#define LAUNCH_SCAN(RR)                                                     \
+  hipLaunchKernelGGL(delta_scan_kernel<RR>, dim3((unsigned)grid), dim3(256), \
+                     0, s, o, qn, kn, vv, decay, beta, ssm, state_slots,     \
+                     qlocs, seq_lens, H, G, dk, dv, col_groups)
+  if (R == 1) LAUNCH_SCAN(1);
+  else if (R == 2) LAUNCH_SCAN(2);
+  else if (R == 4) LAUNCH_SCAN(4);
+  else LAUNCH_SCAN(8);
+#undef LAUNCH_SCAN
 }
 
 extern "C" void mix_delta_out(void* out, long ldo, int out_off, const float* o,

@@ -1,8 +1,10 @@
 // Local (chunked / windowed) paged attention with split key and value sizes.
 //
 //   attn_prep        per-head RMS norm of q and k, rotation of a prefix of
-//                    each head (rotate-half pairing, fp32 angle = position *
-//                    inv_freq[i]), K/V scatter into the paged caches, q out.
+//                    each head (rotate-half pairing; cos and sin of the fp32
+//                    angle position * inv_freq[i] come in a [T, 2*half] table
+//                    made once per step), K/V scatter into the paged caches,
+//                    q out.
 //   local_attention  softmax attention of every new token over the cached
 //                    keys its mask lets it see, times a per-head sigmoid gate.
 //
@@ -22,7 +24,7 @@ __global__ void attn_prep_kernel(
     A* __restrict__ q_out, const A* __restrict__ proj, long ld, int q_off,
     int k_off, int v_off, const float* __restrict__ q_w,
     const float* __restrict__ k_w, float eps,
-    const float* __restrict__ inv_freq, int half, const long* __restrict__ pos,
+    const float* __restrict__ cos_sin, int half,
     const long* __restrict__ slots, A* __restrict__ k_cache,
     A* __restrict__ v_cache, long T, int H, int G, int dk, int dv, int page) {
   extern __shared__ float sm[];  // WPB * dmax floats
@@ -54,7 +56,7 @@ __global__ void attn_prep_kernel(
   const float inv = w ? 1.f / sqrtf(ssq / (float)d + eps) : 1.f;
   __syncthreads();
   const int hf = kind == 2 ? 0 : half;
-  const float p = (float)pos[t];
+  const float* cs = cos_sin + t * 2L * half;  // row t: cos[half] | sin[half]
   A* dst;
   if (kind == 0) {
     dst = q_out + (t * H + head) * (long)dk;
@@ -70,8 +72,7 @@ __global__ void attn_prep_kernel(
       const int fi = i < hf ? i : i - hf;
       const int mate = i < hf ? i + hf : i - hf;
       const float y = buf[mate] * inv * (w ? w[mate] : 1.f);
-      const float a = p * inv_freq[fi];
-      const float c = cosf(a), s = sinf(a);
+      const float c = cs[fi], s = cs[half + fi];
       x = i < hf ? x * c - y * s : x * c + y * s;
     }
     if (valid) stf<A>(dst + i, x);
@@ -161,7 +162,7 @@ __global__ void local_attention_kernel(
 extern "C" void mix_attn_prep(void* q_out, const void* proj, long ld,
                               int q_off, int k_off, int v_off,
                               const float* q_w, const float* k_w, float eps,
-                              const float* inv_freq, int half, const long* pos,
+                              const float* cos_sin, int half,
                               const long* slots, void* k_cache, void* v_cache,
                               long T, int H, int G, int dk, int dv, int page,
                               int f32, hipStream_t s) {
@@ -173,12 +174,12 @@ extern "C" void mix_attn_prep(void* q_out, const void* proj, long ld,
   if (f32)
     hipLaunchKernelGGL(attn_prep_kernel<float>, dim3(grid), dim3(WPB * WAVE),
                        smem, s, (float*)q_out, (const float*)proj, ld, q_off,
-                       k_off, v_off, q_w, k_w, eps, inv_freq, half, pos, slots,
+                       k_off, v_off, q_w, k_w, eps, cos_sin, half, slots,
                        (float*)k_cache, (float*)v_cache, T, H, G, dk, dv, page);
   else
     hipLaunchKernelGGL(attn_prep_kernel<u16>, dim3(grid), dim3(WPB * WAVE),
                        smem, s, (u16*)q_out, (const u16*)proj, ld, q_off,
-                       k_off, v_off, q_w, k_w, eps, inv_freq, half, pos, slots,
+                       k_off, v_off, q_w, k_w, eps, cos_sin, half, slots,
                        (u16*)k_cache, (u16*)v_cache, T, H, G, dk, dv, page);
 }
 

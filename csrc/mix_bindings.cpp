@@ -44,9 +44,8 @@ void mix_gated_norm_residual(float*, const void*, const void*, long, int,
 void mix_scalar_rmsnorm(void*, const float*, const float*, float, long, int,
                         int, hipStream_t);
 void mix_attn_prep(void*, const void*, long, int, int, int, const float*,
-                   const float*, float, const float*, int, const long*,
-                   const long*, void*, void*, long, int, int, int, int, int,
-                   int, hipStream_t);
+                   const float*, float, const float*, int, const long*, void*,
+                   void*, long, int, int, int, int, int, int, hipStream_t);
 void mix_local_attention(void*, long, int, const void*, const void*,
                          const void*, const int*, int, const int*, const int*,
                          const int*, float, int, int, const void*, long, int,
@@ -120,13 +119,12 @@ void scalar_rmsnorm(torch::Tensor out, torch::Tensor x, torch::Tensor gain,
 void attn_prep(torch::Tensor q_out, torch::Tensor proj, long q_off, long k_off,
                long v_off, c10::optional<torch::Tensor> q_w,
                c10::optional<torch::Tensor> k_w, double eps,
-               torch::Tensor inv_freq, torch::Tensor positions,
-               torch::Tensor slots, torch::Tensor k_cache,
+               torch::Tensor cos_sin, torch::Tensor slots,
+               torch::Tensor k_cache,
                torch::Tensor v_cache) {
   CHECK_GPU(proj); CHECK_GPU(q_out); CHECK_CONTIG(q_out);
   CHECK_CONTIG(k_cache); CHECK_CONTIG(v_cache);
-  CHECK_I64(positions); CHECK_I64(slots); CHECK_F32(inv_freq);
-  CHECK_CONTIG(inv_freq);
+  CHECK_I64(slots); CHECK_F32(cos_sin); CHECK_CONTIG(cos_sin);
   const long T = q_out.size(0), H = q_out.size(1), dk = q_out.size(2);
   const long G = k_cache.size(1), page = k_cache.size(2);
   const long dv = v_cache.size(3);
@@ -136,12 +134,13 @@ void attn_prep(torch::Tensor q_out, torch::Tensor proj, long q_off, long k_off,
               k_cache.scalar_type() == proj.scalar_type() &&
               v_cache.scalar_type() == proj.scalar_type(),
               "q, caches and projections must share one dtype");
-  TORCH_CHECK(proj.size(0) == T && positions.numel() == T &&
-              slots.numel() == T, "row mismatch");
+  TORCH_CHECK(proj.size(0) == T && slots.numel() == T &&
+              cos_sin.dim() == 2 && cos_sin.size(0) == T &&
+              cos_sin.size(1) % 2 == 0, "row mismatch");
   check_proj(proj, q_off, H * dk, "q");
   check_proj(proj, k_off, G * dk, "k");
   check_proj(proj, v_off, G * dv, "v");
-  const long half = inv_freq.numel();
+  const long half = cos_sin.size(1) / 2;
   TORCH_CHECK(2 * half <= dk, "rotated prefix longer than the head");
   const float* qw = nullptr; const float* kw = nullptr;
   if (q_w.has_value()) {
@@ -154,8 +153,7 @@ void attn_prep(torch::Tensor q_out, torch::Tensor proj, long q_off, long k_off,
   }
   mix_attn_prep(q_out.data_ptr(), proj.data_ptr(), proj.stride(0), (int)q_off,
                 (int)k_off, (int)v_off, qw, kw, (float)eps,
-                inv_freq.data_ptr<float>(), (int)half,
-                positions.data_ptr<long>(), slots.data_ptr<long>(),
+                cos_sin.data_ptr<float>(), (int)half, slots.data_ptr<long>(),
                 k_cache.data_ptr(), v_cache.data_ptr(), T, (int)H, (int)G,
                 (int)dk, (int)dv, (int)page, act_kind(proj), cur_stream());
 }

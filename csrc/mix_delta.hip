@@ -30,39 +30,20 @@ __device__ __forceinline__ int chan_col(int c, int Cq, int q_off, int k_off,
 template <typename A>
 __global__ void delta_prep_kernel(
     float* __restrict__ qn, float* __restrict__ kn, float* __restrict__ vv,
-    float* __restrict__ decay, float* __restrict__ beta,
     const A* __restrict__ proj, long ld, int q_off, int k_off, int v_off,
-    int b_off, int a1_off, const float* __restrict__ conv_w, int taps,
-    const float* __restrict__ a2, int rank, const float* __restrict__ dt_bias,
-    const float* __restrict__ a_log, const float* __restrict__ conv_state,
+    const float* __restrict__ conv_w, int taps,
+    const float* __restrict__ conv_state,
     const int* __restrict__ state_slots, const int* __restrict__ qlocs,
     const int* __restrict__ seq_lens, const int* __restrict__ token_seq,
     long T, int H, int G, int dk, int dv) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int wid = threadIdx.x / WAVE;
-  const int units = 2 * G + 2 * H;
+  const int units = 2 * G + H;
   const long u = (long)blockIdx.x * WPB + wid;
   if (u >= T * units) return;
   const long t = u / units;
   const int j = (int)(u - t * units);
   const int Cq = G * dk, C = 2 * Cq + H * dv;
-
-  if (j >= 2 * G + H) {  // decay + beta of head h
-    const int h = j - 2 * G - H;
-    const A* a1 = proj + t * ld + a1_off;
-    const float rate = expf(a_log[h]);
-    const long HD = (long)H * dk;
-    for (int i = lane; i < dk; i += WAVE) {
-      // a2 is stored transposed [rank, H*dk]: lanes read consecutive floats
-      const float* w = a2 + (long)h * dk + i;
-      float a = dt_bias[h * dk + i];
-      for (int r = 0; r < rank; ++r) a += w[r * HD] * ldf<A>(a1 + r);
-      decay[(t * H + h) * (long)dk + i] = expf(-rate * softplus_f(a));
-    }
-    if (lane == 0)
-      beta[t * H + h] = sigmoid_f(ldf<A>(proj + t * ld + b_off + h));
-    return;
-  }
 
   // filter + silu of one q, k or v head
   const int kind = j < G ? 0 : (j < 2 * G ? 1 : 2);
@@ -105,6 +86,80 @@ __global__ void delta_prep_kernel(
                                       : vv + (t * H + head) * (long)dv);
   k = 0;
   for (int i = lane; i < d; i += WAVE, ++k) dst[i] = y[k] * f;
+}
+
+// ---- low-rank gates ---------------------------------------------------------
+// Both gate kernels evaluate act(W2 (W1 h) + bias) where W1 h (`rank` numbers
+// a token) is a section of the merged projection and W2 arrives transposed
+// [rank, rows]. A wave owns GT consecutive tokens and one head: a lane keeps
+// the W2 column of its output channel in registers across those tokens, the
+// token's `rank` inputs sit one per lane and reach the FMAs through readlane
+// (scalar operands), so the inner loop issues no loads at all.
+#define GT 8     // tokens per wave
+#define RMAX 32  // W2 rows held per pass
+
+__device__ __forceinline__ float lane_bcast(float v, int src) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src));
+}
+
+// acc[tt] += sum_r w2t[(r0 + r) * stride + col] * in[t_base + tt][r0 + r]
+template <typename A>
+__device__ __forceinline__ void low_rank_acc(
+    float (&acc)[GT], const float* __restrict__ w2t, long stride, long col,
+    bool col_ok, int rank, const A* __restrict__ in, long ld, long t_base,
+    long T, int lane) {
+  for (int r0 = 0; r0 < rank; r0 += RMAX) {
+    float w[RMAX];
+#pragma unroll
+    for (int r = 0; r < RMAX; ++r)
+      w[r] = (col_ok && r0 + r < rank) ? w2t[(long)(r0 + r) * stride + col] : 0.f;
+#pragma unroll
+    for (int tt = 0; tt < GT; ++tt) {
+      const long t = t_base + tt;
+      if (t >= T) break;  // wave-uniform
+      const float x = (lane < RMAX && r0 + lane < rank)
+                          ? ldf<A>(in + t * ld + r0 + lane) : 0.f;
+      float a = 0.f;
+#pragma unroll
+      for (int r = 0; r < RMAX; ++r) a += w[r] * lane_bcast(x, r);
+      acc[tt] += a;
+    }
+  }
+}
+
+// decay[t,h,i] = exp(-exp(a_log[h]) * softplus(a2 a1 + dt_bias)), beta[t,h] =
+// sigmoid(b section). grid (token groups, H).
+template <typename A>
+__global__ void delta_gates_kernel(
+    float* __restrict__ decay, float* __restrict__ beta,
+    const A* __restrict__ proj, long ld, int b_off, int a1_off,
+    const float* __restrict__ a2t, int rank, const float* __restrict__ dt_bias,
+    const float* __restrict__ a_log, long T, int H, int dk) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int wid = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+  const int h = blockIdx.y;
+  const long t_base = ((long)blockIdx.x * WPB + wid) * GT;
+  if (t_base >= T) return;
+  const float rate = expf(a_log[h]);
+  const long HD = (long)H * dk;
+  for (int k0 = 0; k0 < dk; k0 += WAVE) {
+    const int i = k0 + lane;
+    const bool in = i < dk;
+    float acc[GT];
+    const float bias = in ? dt_bias[h * dk + i] : 0.f;
+#pragma unroll
+    for (int tt = 0; tt < GT; ++tt) acc[tt] = bias;
+    low_rank_acc<A>(acc, a2t, HD, (long)h * dk + i, in, rank, proj + a1_off, ld,
+                    t_base, T, lane);
+#pragma unroll
+    for (int tt = 0; tt < GT; ++tt)
+      if (in && t_base + tt < T)
+        decay[((t_base + tt) * H + h) * (long)dk + i] =
+            expf(-rate * softplus_f(acc[tt]));
+  }
+  if (lane < GT && t_base + lane < T)
+    beta[(t_base + lane) * H + h] =
+        sigmoid_f(ldf<A>(proj + (t_base + lane) * ld + b_off + h));
 }
 
 // one thread per (sequence, channel): new history = last taps-1 raw inputs
@@ -268,33 +323,51 @@ __global__ void __launch_bounds__(256) delta_scan_kernel(
   }
 }
 
+// out[t, out_off + h*dv + c] = out_scale * o[t,h,c] / rms(o[t,h,:]) * w[c] *
+// sigmoid(g2 g1)[h*dv + c]. grid (token groups, H); a wave owns GT tokens.
 template <typename A>
 __global__ void delta_out_kernel(A* __restrict__ out, long ldo, int out_off,
                                  const float* __restrict__ o,
                                  const float* __restrict__ norm_w,
                                  const A* __restrict__ proj, long ld,
-                                 int g1_off, const float* __restrict__ g2,
+                                 int g1_off, const float* __restrict__ g2t,
                                  int rank, float eps, float out_scale, long T,
                                  int H, int dv) {
   const int lane = threadIdx.x & (WAVE - 1);
-  const long u = (long)blockIdx.x * WPB + threadIdx.x / WAVE;
-  if (u >= T * H) return;
-  const long t = u / H;
-  const int h = (int)(u - t * H);
-  const float* orow = o + u * dv;
-  float ssq = 0.f;
-  for (int c = lane; c < dv; c += WAVE) ssq += orow[c] * orow[c];
-  ssq = wave_sum_f32(ssq);
-  const float inv = out_scale / sqrtf(ssq / (float)dv + eps);
-  const A* g1 = proj + t * ld + g1_off;
+  const int wid = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+  const int h = blockIdx.y;
+  const long t_base = ((long)blockIdx.x * WPB + wid) * GT;
+  if (t_base >= T) return;
+  float inv[GT];
+#pragma unroll
+  for (int tt = 0; tt < GT; ++tt) {
+    inv[tt] = 0.f;
+    const long t = t_base + tt;
+    if (t >= T) break;
+    const float* orow = o + (t * H + h) * (long)dv;
+    float ssq = 0.f;
+    for (int c = lane; c < dv; c += WAVE) ssq += orow[c] * orow[c];
+    ssq = wave_sum_f32(ssq);
+    inv[tt] = out_scale / sqrtf(ssq / (float)dv + eps);
+  }
   const long HV = (long)H * dv;
-  for (int c = lane; c < dv; c += WAVE) {
-    // g2 is stored transposed [rank, H*dv]
-    const float* w = g2 + (long)h * dv + c;
-    float a = 0.f;
-    for (int r = 0; r < rank; ++r) a += w[r * HV] * ldf<A>(g1 + r);
-    stf<A>(out + t * ldo + out_off + (long)h * dv + c,
-           orow[c] * inv * norm_w[c] * sigmoid_f(a));
+  for (int k0 = 0; k0 < dv; k0 += WAVE) {
+    const int c = k0 + lane;
+    const bool in = c < dv;
+    float acc[GT];
+#pragma unroll
+    for (int tt = 0; tt < GT; ++tt) acc[tt] = 0.f;
+    low_rank_acc<A>(acc, g2t, HV, (long)h * dv + c, in, rank, proj + g1_off, ld,
+                    t_base, T, lane);
+    const float wn = in ? norm_w[c] : 0.f;
+#pragma unroll
+    for (int tt = 0; tt < GT; ++tt) {
+      const long t = t_base + tt;
+      if (in && t < T)
+        stf<A>(out + t * ldo + out_off + (long)h * dv + c,
+               o[(t * H + h) * (long)dv + c] * inv[tt] * wn *
+                   sigmoid_f(acc[tt]));
+    }
   }
 }
 
@@ -306,18 +379,21 @@ extern "C" void mix_delta_prep(
     const int* state_slots, const int* qlocs, const int* seq_lens,
     const int* token_seq, long T, int S, int H, int G, int dk, int dv, int f32,
     hipStream_t s) {
-  const long units = T * (2 * G + 2 * H);
+  const long units = T * (2 * G + H);
   const int grid = (int)((units + WPB - 1) / WPB);
   if (grid == 0) return;
+  const dim3 ggrid((unsigned)((T + WPB * GT - 1) / (WPB * GT)), (unsigned)H);
   const int Cq = G * dk, C = 2 * Cq + H * dv;
   const long su = (long)S * C;
   const int sgrid = (int)((su + 255) / 256);
   if (f32) {
     hipLaunchKernelGGL(delta_prep_kernel<float>, dim3(grid), dim3(WPB * WAVE),
-                       0, s, qn, kn, vv, decay, beta, (const float*)proj, ld,
-                       q_off, k_off, v_off, b_off, a1_off, conv_w, taps, a2,
-                       rank, dt_bias, a_log, conv_state, state_slots, qlocs,
+                       0, s, qn, kn, vv, (const float*)proj, ld, q_off, k_off,
+                       v_off, conv_w, taps, conv_state, state_slots, qlocs,
                        seq_lens, token_seq, T, H, G, dk, dv);
+    hipLaunchKernelGGL(delta_gates_kernel<float>, ggrid, dim3(WPB * WAVE), 0, s,
+                       decay, beta, (const float*)proj, ld, b_off, a1_off, a2,
+                       rank, dt_bias, a_log, T, H, dk);
     if (taps > 1)
       hipLaunchKernelGGL(conv_state_update_kernel<float>, dim3(sgrid),
                          dim3(256), 0, s, conv_state, (const float*)proj, ld,
@@ -325,10 +401,12 @@ extern "C" void mix_delta_prep(
                          seq_lens, S, Cq, C);
   } else {
     hipLaunchKernelGGL(delta_prep_kernel<u16>, dim3(grid), dim3(WPB * WAVE), 0,
-                       s, qn, kn, vv, decay, beta, (const u16*)proj, ld, q_off,
-                       k_off, v_off, b_off, a1_off, conv_w, taps, a2, rank,
-                       dt_bias, a_log, conv_state, state_slots, qlocs,
-                       seq_lens, token_seq, T, H, G, dk, dv);
+                       s, qn, kn, vv, (const u16*)proj, ld, q_off, k_off, v_off,
+                       conv_w, taps, conv_state, state_slots, qlocs, seq_lens,
+                       token_seq, T, H, G, dk, dv);
+    hipLaunchKernelGGL(delta_gates_kernel<u16>, ggrid, dim3(WPB * WAVE), 0, s,
+                       decay, beta, (const u16*)proj, ld, b_off, a1_off, a2,
+                       rank, dt_bias, a_log, T, H, dk);
     if (taps > 1)
       hipLaunchKernelGGL(conv_state_update_kernel<u16>, dim3(sgrid), dim3(256),
                          0, s, conv_state, (const u16*)proj, ld, q_off, k_off,
@@ -364,16 +442,15 @@ extern "C" void mix_delta_out(void* out, long ldo, int out_off, const float* o,
                               int g1_off, const float* g2, int rank, float eps,
                               float out_scale, long T, int H, int dv, int f32,
                               hipStream_t s) {
-  const long units = T * H;
-  const int grid = (int)((units + WPB - 1) / WPB);
-  if (grid == 0) return;
+  if (T == 0) return;
+  const dim3 grid((unsigned)((T + WPB * GT - 1) / (WPB * GT)), (unsigned)H);
   if (f32)
-    hipLaunchKernelGGL(delta_out_kernel<float>, dim3(grid), dim3(WPB * WAVE),
+    hipLaunchKernelGGL(delta_out_kernel<float>, grid, dim3(WPB * WAVE),
                        0, s, (float*)out, ldo, out_off, o, norm_w,
                        (const float*)proj, ld, g1_off, g2, rank, eps,
                        out_scale, T, H, dv);
   else
-    hipLaunchKernelGGL(delta_out_kernel<u16>, dim3(grid), dim3(WPB * WAVE), 0,
+    hipLaunchKernelGGL(delta_out_kernel<u16>, grid, dim3(WPB * WAVE), 0,
                        s, (u16*)out, ldo, out_off, o, norm_w,
                        (const u16*)proj, ld, g1_off, g2, rank, eps, out_scale,
                        T, H, dv);

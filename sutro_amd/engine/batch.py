@@ -2,7 +2,7 @@
 
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import List, Optional
 
 import torch
@@ -48,3 +48,5 @@ class ForwardBatch:
     # models with per-sequence recurrent state / per-token sequence lookups
     state_slots: Optional[torch.Tensor] = None  # [S] int32 state slot per seq
     token_seq: Optional[torch.Tensor] = None    # [T] int32 seq index per row
+    # per-step scratch shared by a model's layers (e.g. rotation tables)
+    aux: dict = field(default_factory=dict)

@@ -111,12 +111,21 @@ class LocalAttention(nn.Module):
                 out_off: int, out_scale: float) -> None:
         s = self.spec
         kc, vc = kv.k_cache[self.layer_idx], kv.v_cache[self.layer_idx]
+        cos_sin = None
+        if proj.is_cuda:
+            # one cos/sin table per step and kind of rotation, shared by layers
+            key = ("rope", s.rot_dims, s.rot_base)
+            cos_sin = fb.aux.get(key)
+            if cos_sin is None:
+                cos_sin = fb.aux[key] = hops.rope_table(fb.positions,
+                                                        self.inv_freq)
         q = hops.attn_prep(
             proj, off[tag + "q"], off[tag + "k"], off[tag + "v"], s.heads,
             s.kv_heads, s.dim, s.vdim,
             self.q_norm if s.qk_norm else None,
             self.k_norm if s.qk_norm else None,
-            self.eps, self.inv_freq, fb.positions, fb.slot_mapping, kc, vc)
+            self.eps, self.inv_freq, fb.positions, fb.slot_mapping, kc, vc,
+            cos_sin=cos_sin)
         hops.local_attention(
             q, kc, vc, fb.block_tables, fb.seq_lens, fb.query_start_locs,
             s.scale, s.chunk, s.window, proj,

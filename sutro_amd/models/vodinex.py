@@ -198,6 +198,10 @@ class VodinexModel(nn.Module):
 
     @torch.no_grad()
     def forward(self, fb: ForwardBatch, kv: PagedKVCache) -> torch.Tensor:
+        # per-step scratch (rotation tables) is rebuilt on every pass: a batch
+        # object that is run again (graph warm-up, then capture) must not keep
+        # tables of the earlier pass
+        fb.aux.clear()
         h = self.embed_tokens(fb.input_ids)
         if h.dtype == torch.float32:
             x = h = h.clone()

@@ -67,14 +67,23 @@ def scalar_rmsnorm(x, gain, eps: float, out_dtype: torch.dtype):
     return torch_ref.scalar_rmsnorm(x, gain, eps, out_dtype)
 
 
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+    """fp32 [T, 2*half]: cos | sin of the fp32 angle position * inv_freq.
+    One table serves every layer of a step that rotates alike."""
+    ang = positions.to(torch.float32).unsqueeze(1) * inv_freq.unsqueeze(0)
+    return torch.cat([ang.cos(), ang.sin()], dim=1).contiguous()
+
+
 def attn_prep(proj, q_off, k_off, v_off, H, G, dk, dv, q_norm_w, k_norm_w,
-              eps, inv_freq, positions, slot_mapping, k_cache, v_cache):
+              eps, inv_freq, positions, slot_mapping, k_cache, v_cache,
+              cos_sin=None):
     if proj.is_cuda:
         q = torch.empty((proj.shape[0], H, dk), dtype=proj.dtype,
                         device=proj.device)
+        if cos_sin is None:
+            cos_sin = rope_table(positions, inv_freq)
         _mix().attn_prep(q, proj, q_off, k_off, v_off, q_norm_w, k_norm_w,
-                         eps, inv_freq, positions, slot_mapping, k_cache,
-                         v_cache)
+                         eps, cos_sin, slot_mapping, k_cache, v_cache)
         return q
     return torch_ref.attn_prep(proj, q_off, k_off, v_off, H, G, dk, dv,
                                q_norm_w, k_norm_w, eps, inv_freq, positions,

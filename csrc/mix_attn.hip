@@ -19,6 +19,14 @@
 
 #define WPB 4  // waves per block
 
+#define UPW 4   // (token, head) units per wave
+#define DPL 4   // elements per lane and unit (head sizes up to 64 * DPL)
+
+// A wave handles UPW consecutive units (a unit = one q, k or v head of one
+// token): the global loads of all its units are issued before any of them is
+// reduced, so their latencies overlap. The normalised head passes through a
+// wave-private LDS row to bring rotation partners (i, i + half) together;
+// LDS operations of one wave execute in order, so no barrier is needed.
 template <typename A>
 __global__ void attn_prep_kernel(
     A* __restrict__ q_out, const A* __restrict__ proj, long ld, int q_off,
@@ -33,50 +41,166 @@ __global__ void attn_prep_kernel(
   const int dmax = dk > dv ? dk : dv;
   float* buf = sm + wid * dmax;
   const int units = H + 2 * G;
-  const long u = (long)blockIdx.x * WPB + wid;
-  const bool valid = u < T * units;
+  const long total = T * units;
+  const long u0 = ((long)blockIdx.x * WPB + wid) * UPW;
+
+  float x[UPW][DPL];
+#pragma unroll
+  for (int n = 0; n < UPW; ++n) {
+    const long u = u0 + n;
+    const long t = u < total ? u / units : 0;
+    const int j = u < total ? (int)(u - t * units) : 0;
+    const int kind = j < H ? 0 : (j < H + G ? 1 : 2);
+    const int head = kind == 0 ? j : (kind == 1 ? j - H : j - H - G);
+    const int d = kind == 2 ? dv : dk;
+    const A* src = proj + t * ld +
+                   (kind == 0 ? q_off : (kind == 1 ? k_off : v_off)) +
+                   (long)head * d;
+#pragma unroll
+    for (int k = 0; k < DPL; ++k) {
+      const int i = lane + k * (int)WAVE;
+      x[n][k] = i < d ? ldf<A>(src + i) : 0.f;
+    }
+  }
+#pragma unroll
+  for (int n = 0; n < UPW; ++n) {
+    const long u = u0 + n;
+    if (u >= total) break;  // wave-uniform
+    const long t = u / units;
+    const int j = (int)(u - t * units);
+    const int kind = j < H ? 0 : (j < H + G ? 1 : 2);
+    const int head = kind == 0 ? j : (kind == 1 ? j - H : j - H - G);
+    const int d = kind == 2 ? dv : dk;
+    const float* w = kind == 0 ? q_w : (kind == 1 ? k_w : nullptr);
+    float ssq = 0.f;
+#pragma unroll
+    for (int k = 0; k < DPL; ++k) ssq += x[n][k] * x[n][k];
+    ssq = wave_sum_f32(ssq);
+    const float inv = w ? 1.f / sqrtf(ssq / (float)d + eps) : 1.f;
+#pragma unroll
+    for (int k = 0; k < DPL; ++k) {
+      const int i = lane + k * (int)WAVE;
+      if (i < d) {
+        x[n][k] *= inv * (w ? w[i] : 1.f);
+        buf[i] = x[n][k];
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+    const int hf = kind == 2 ? 0 : half;
+    const float* cs = cos_sin + t * 2L * half;  // row t: cos[half] | sin[half]
+    A* dst;
+    if (kind == 0) {
+      dst = q_out + (t * H + head) * (long)dk;
+    } else {
+      const long slot = slots[t];
+      const long blk = slot / page, off = slot - blk * page;
+      dst = (kind == 1 ? k_cache : v_cache) +
+            ((blk * G + head) * page + off) * (long)d;
+    }
+#pragma unroll
+    for (int k = 0; k < DPL; ++k) {
+      const int i = lane + k * (int)WAVE;
+      if (i >= d) continue;
+      float v = x[n][k];
+      if (i < 2 * hf) {
+        const int fi = i < hf ? i : i - hf;
+        const float y = buf[i < hf ? i + hf : i - hf];
+        const float c = cs[fi], sn = cs[half + fi];
+        v = i < hf ? v * c - y * sn : v * c + y * sn;
+      }
+      stf<A>(dst + i, v);
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+// bf16 fast path of attn_prep: a group of GS lanes owns one unit, lane gl its
+// 8-element chunk gl (one 16-byte load and store a lane). The norm reduces
+// over the group by xor-shuffles; the rotation partner chunk (gl +- half/8)
+// arrives by lane shuffles. Needs dk, dv, half and all offsets to be multiples
+// of 8; other shapes and fp32 take the generic kernel above.
+template <int GS>
+__global__ void attn_prep_vec_kernel(
+    u16* __restrict__ q_out, const u16* __restrict__ proj, long ld, int q_off,
+    int k_off, int v_off, const float* __restrict__ q_w,
+    const float* __restrict__ k_w, float eps,
+    const float* __restrict__ cos_sin, int half,
+    const long* __restrict__ slots, u16* __restrict__ k_cache,
+    u16* __restrict__ v_cache, long T, int H, int G, int dk, int dv, int page) {
+  constexpr int UPWV = 64 / GS;
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int wid = threadIdx.x / WAVE;
+  const int gi = lane / GS, gl = lane % GS;
+  const int units = H + 2 * G;
+  const long total = T * units;
+  const long u = ((long)blockIdx.x * WPB + wid) * UPWV + gi;
+  const bool valid = u < total;
   const long t = valid ? u / units : 0;
   const int j = valid ? (int)(u - t * units) : 0;
-  // unit kind: 0 = q head, 1 = k head, 2 = v head
   const int kind = j < H ? 0 : (j < H + G ? 1 : 2);
   const int head = kind == 0 ? j : (kind == 1 ? j - H : j - H - G);
   const int d = kind == 2 ? dv : dk;
-  const A* src = proj + t * ld +
-                 (kind == 0 ? q_off : (kind == 1 ? k_off : v_off)) +
-                 (long)head * d;
-  const float* w = kind == 0 ? q_w : (kind == 1 ? k_w : nullptr);
-
-  float ssq = 0.f;
-  for (int i = lane; i < d; i += WAVE) {
-    const float x = ldf<A>(src + i);
-    buf[i] = x;
-    ssq += x * x;
+  const int c0 = gl * 8;
+  const bool act = valid && c0 < d;
+  const u16* src = proj + t * ld +
+                   (kind == 0 ? q_off : (kind == 1 ? k_off : v_off)) +
+                   (long)head * d + c0;
+  float x[8];
+  {
+    u16x8 raw = (u16x8)(0);
+    if (act) raw = *(const u16x8*)src;
+    bf8_to_f32(raw, x);
   }
-  ssq = wave_sum_f32(ssq);
-  const float inv = w ? 1.f / sqrtf(ssq / (float)d + eps) : 1.f;
-  __syncthreads();
-  const int hf = kind == 2 ? 0 : half;
-  const float* cs = cos_sin + t * 2L * half;  // row t: cos[half] | sin[half]
-  A* dst;
+  float ssq = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ssq += x[e] * x[e];
+#pragma unroll
+  for (int off = GS / 2; off > 0; off >>= 1) ssq += __shfl_xor(ssq, off, WAVE);
+  const float* w = kind == 0 ? q_w : (kind == 1 ? k_w : nullptr);
+  if (w && act) {
+    const float inv = 1.f / sqrtf(ssq / (float)d + eps);
+    const f32x4 w0 = *(const f32x4*)(w + c0), w1 = *(const f32x4*)(w + c0 + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      x[e] *= inv * w0[e];
+      x[e + 4] *= inv * w1[e];
+    }
+  }
+  const int hc = half / 8;  // chunks in half of the rotated prefix
+  if (hc > 0) {             // uniform: every lane takes part in the shuffles
+    const bool rot = kind != 2 && c0 < 2 * half;
+    const bool first = c0 < half;
+    const int partner = rot ? (first ? lane + hc : lane - hc) : lane;
+    float y[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = __shfl(x[e], partner, WAVE);
+    if (rot && act) {
+      const float* cs = cos_sin + t * 2L * half + (first ? c0 : c0 - half);
+      const f32x4 ca = *(const f32x4*)cs, cb = *(const f32x4*)(cs + 4);
+      const f32x4 sa = *(const f32x4*)(cs + half),
+                  sb = *(const f32x4*)(cs + half + 4);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float c = e < 4 ? ca[e & 3] : cb[e & 3];
+        const float sn = e < 4 ? sa[e & 3] : sb[e & 3];
+        x[e] = first ? x[e] * c - y[e] * sn : x[e] * c + y[e] * sn;
+      }
+    }
+  }
+  if (!act) return;
+  u16* dst;
   if (kind == 0) {
-    dst = q_out + (t * H + head) * (long)dk;
+    dst = q_out + (t * H + head) * (long)dk + c0;
   } else {
     const long slot = slots[t];
     const long blk = slot / page, off = slot - blk * page;
     dst = (kind == 1 ? k_cache : v_cache) +
-          ((blk * G + head) * page + off) * (long)d;
+          ((blk * G + head) * page + off) * (long)d + c0;
   }
-  for (int i = lane; i < d; i += WAVE) {
-    float x = buf[i] * inv * (w ? w[i] : 1.f);
-    if (i < 2 * hf) {
-      const int fi = i < hf ? i : i - hf;
-      const int mate = i < hf ? i + hf : i - hf;
-      const float y = buf[mate] * inv * (w ? w[mate] : 1.f);
-      const float c = cs[fi], s = cs[half + fi];
-      x = i < hf ? x * c - y * s : x * c + y * s;
-    }
-    if (valid) stf<A>(dst + i, x);
-  }
+  u16x8 o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = f2bf(x[e]);
+  *(u16x8*)dst = o;
 }
 
 // NV = value columns per lane (dv <= 64 * NV)
@@ -166,11 +290,30 @@ extern "C" void mix_attn_prep(void* q_out, const void* proj, long ld,
                               const long* slots, void* k_cache, void* v_cache,
                               long T, int H, int G, int dk, int dv, int page,
                               int f32, hipStream_t s) {
-  const long units = T * (H + 2 * G);
+  const long units = (T * (H + 2 * G) + UPW - 1) / UPW;
   const int grid = (int)((units + WPB - 1) / WPB);
   const int dmax = dk > dv ? dk : dv;
   const size_t smem = (size_t)WPB * dmax * sizeof(float);
   if (grid == 0) return;
+  const int dm8 = (dmax + 7) / 8;
+  if (!f32 && dk % 8 == 0 && dv % 8 == 0 && half % 8 == 0 && ld % 8 == 0 &&
+      q_off % 8 == 0 && k_off % 8 == 0 && v_off % 8 == 0 && dm8 <= 32) {
+    const int GS = dm8 <= 4 ? 4 : (dm8 <= 8 ? 8 : (dm8 <= 16 ? 16 : 32));
+    const long tot = T * (H + 2 * G);
+    const long waves = (tot + 64 / GS - 1) / (64 / GS);
+    const int vgrid = (int)((waves + WPB - 1) / WPB);
+#define LAUNCH_PV(GG)                                                         \
+  hipLaunchKernelGGL(attn_prep_vec_kernel<GG>, dim3(vgrid), dim3(WPB * WAVE), \
+                     0, s, (u16*)q_out, (const u16*)proj, ld, q_off, k_off,   \
+                     v_off, q_w, k_w, eps, cos_sin, half, slots,              \
+                     (u16*)k_cache, (u16*)v_cache, T, H, G, dk, dv, page)
+    if (GS == 4) LAUNCH_PV(4);
+    else if (GS == 8) LAUNCH_PV(8);
+    else if (GS == 16) LAUNCH_PV(16);
+    else LAUNCH_PV(32);
+#undef LAUNCH_PV
+    return;
+  }
   if (f32)
     hipLaunchKernelGGL(attn_prep_kernel<float>, dim3(grid), dim3(WPB * WAVE),
                        smem, s, (float*)q_out, (const float*)proj, ld, q_off,

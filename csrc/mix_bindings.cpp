@@ -57,7 +57,8 @@ int mix_local_attention_mfma(void*, long, int, const void*, const void*,
                              int, int, const void*, long, int, float, int, int,
                              int, int, int, hipStream_t);
 void mix_delta_prep(float*, float*, float*, float*, float*, const void*, long,
-                    int, int, int, int, int, const float*, int, const float*,
+                    int, int, int, int, int, const float*, const float*, int,
+                    const float*,
                     int, const float*, const float*, float*, const int*,
                     const int*, const int*, const int*, long, int, int, int,
                     int, int, int, hipStream_t);
@@ -142,6 +143,7 @@ void attn_prep(torch::Tensor q_out, torch::Tensor proj, long q_off, long k_off,
   check_proj(proj, v_off, G * dv, "v");
   const long half = cos_sin.size(1) / 2;
   TORCH_CHECK(2 * half <= dk, "rotated prefix longer than the head");
+  TORCH_CHECK(dk <= 256 && dv <= 256, "head sizes above 256 are unsupported");
   const float* qw = nullptr; const float* kw = nullptr;
   if (q_w.has_value()) {
     CHECK_F32(*q_w); TORCH_CHECK(q_w->numel() == dk, "q norm size");
@@ -223,8 +225,16 @@ void delta_prep(torch::Tensor qn, torch::Tensor kn, torch::Tensor v,
                 torch::Tensor conv_w, torch::Tensor a2, torch::Tensor dt_bias,
                 torch::Tensor a_log, torch::Tensor conv_state,
                 torch::Tensor state_slots, torch::Tensor qlocs,
-                torch::Tensor seq_lens, torch::Tensor token_seq) {
+                torch::Tensor seq_lens, torch::Tensor token_seq,
+                c10::optional<torch::Tensor> conv_wt) {
   CHECK_GPU(proj);
+  const float* wt = nullptr;
+  if (conv_wt.has_value()) {  // the filter transposed: [taps, channels]
+    CHECK_F32(*conv_wt); CHECK_CONTIG(*conv_wt);
+    TORCH_CHECK(conv_wt->dim() == 2 && conv_wt->size(0) == conv_w.size(1) &&
+                conv_wt->size(1) == conv_w.size(0), "transposed filter shape");
+    wt = conv_wt->data_ptr<float>();
+  }
   CHECK_F32(qn); CHECK_F32(kn); CHECK_F32(v); CHECK_F32(decay); CHECK_F32(beta);
   CHECK_CONTIG(qn); CHECK_CONTIG(kn); CHECK_CONTIG(v); CHECK_CONTIG(decay);
   CHECK_CONTIG(beta);
@@ -260,7 +270,7 @@ void delta_prep(torch::Tensor qn, torch::Tensor kn, torch::Tensor v,
                  v.data_ptr<float>(), decay.data_ptr<float>(),
                  beta.data_ptr<float>(), proj.data_ptr(), proj.stride(0),
                  (int)q_off, (int)k_off, (int)v_off, (int)b_off, (int)a1_off,
-                 conv_w.data_ptr<float>(), (int)taps, a2.data_ptr<float>(),
+                 conv_w.data_ptr<float>(), wt, (int)taps, a2.data_ptr<float>(),
                  (int)rank, dt_bias.data_ptr<float>(), a_log.data_ptr<float>(),
                  conv_state.data_ptr<float>(), state_slots.data_ptr<int>(),
                  qlocs.data_ptr<int>(), seq_lens.data_ptr<int>(),
@@ -331,7 +341,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("gate_off"), py::arg("out_scale"),
         py::arg("tile_seq") = c10::nullopt, py::arg("tile_q0") = c10::nullopt,
         py::arg("prefill_rows") = 0);
-  m.def("delta_prep", &delta_prep, "delta-rule inputs: filters, norms, gates");
+  m.def("delta_prep", &delta_prep, "delta-rule inputs: filters, norms, gates",
+        py::arg("qn"), py::arg("kn"), py::arg("v"), py::arg("decay"),
+        py::arg("beta"), py::arg("proj"), py::arg("q_off"), py::arg("k_off"),
+        py::arg("v_off"), py::arg("b_off"), py::arg("a1_off"),
+        py::arg("conv_w"), py::arg("a2"), py::arg("dt_bias"), py::arg("a_log"),
+        py::arg("conv_state"), py::arg("state_slots"), py::arg("qlocs"),
+        py::arg("seq_lens"), py::arg("token_seq"),
+        py::arg("conv_wt") = c10::nullopt);
   m.def("delta_scan", &delta_scan, "gated delta rule over new tokens");
   m.def("delta_out", &delta_out, "per-head norm + low-rank gate of the read-out");
 }

@@ -20,6 +20,7 @@
 #include "mix_common.h"
 
 #define WPB 4
+#define PT 8   // tokens per wave in delta_prep
 
 // merged channel c (q | k | v order) -> column of the projection buffer
 __device__ __forceinline__ int chan_col(int c, int Cq, int q_off, int k_off,
@@ -39,12 +40,12 @@ __global__ void delta_prep_kernel(
   const int lane = threadIdx.x & (WAVE - 1);
   const int wid = threadIdx.x / WAVE;
   const int units = 2 * G + H;
-  const long u = (long)blockIdx.x * WPB + wid;
-  if (u >= T * units) return;
-  const long t = u / units;
-  const int j = (int)(u - t * units);
+  // a wave owns one head unit and PT consecutive tokens
+  const long wv = (long)blockIdx.x * WPB + wid;
+  const long tg = wv / units;
+  const int j = (int)(wv - tg * units);
   const int Cq = G * dk, C = 2 * Cq + H * dv;
-
+  for (long t = tg * PT; t < T && t < (tg + 1) * PT; ++t) {
   // filter + silu of one q, k or v head
   const int kind = j < G ? 0 : (j < 2 * G ? 1 : 2);
   const int head = kind == 0 ? j : (kind == 1 ? j - G : j - 2 * G);
@@ -86,6 +87,92 @@ __global__ void delta_prep_kernel(
                                       : vv + (t * H + head) * (long)dv);
   k = 0;
   for (int i = lane; i < d; i += WAVE, ++k) dst[i] = y[k] * f;
+  }  // tokens of this wave
+}
+
+// bf16 fast path of delta_prep: a group of GS lanes owns one (token, head)
+// unit, lane gl its 8-channel chunk (16-byte loads of the raw rows, float4
+// loads of the transposed filter [taps, C] and of the history, float4
+// stores). Needs dk, dv and all offsets to be multiples of 8.
+template <int GS>
+__global__ void delta_prep_vec_kernel(
+    float* __restrict__ qn, float* __restrict__ kn, float* __restrict__ vv,
+    const u16* __restrict__ proj, long ld, int q_off, int k_off, int v_off,
+    const float* __restrict__ conv_wt, int taps,
+    const float* __restrict__ conv_state,
+    const int* __restrict__ state_slots, const int* __restrict__ qlocs,
+    const int* __restrict__ seq_lens, const int* __restrict__ token_seq,
+    long T, int H, int G, int dk, int dv) {
+  constexpr int UPWV = 64 / GS;
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int wid = threadIdx.x / WAVE;
+  const int gi = lane / GS, gl = lane % GS;
+  const int units = 2 * G + H;
+  const long total = T * units;
+  const long u = ((long)blockIdx.x * WPB + wid) * UPWV + gi;
+  const bool valid = u < total;
+  const long t = valid ? u / units : 0;
+  const int j = valid ? (int)(u - t * units) : 0;
+  const int Cq = G * dk, C = 2 * Cq + H * dv;
+  const int kind = j < G ? 0 : (j < 2 * G ? 1 : 2);
+  const int head = kind == 0 ? j : (kind == 1 ? j - G : j - 2 * G);
+  const int d = kind == 2 ? dv : dk;
+  const int c0 = gl * 8;
+  const bool act = valid && c0 < d;
+  const int c = (kind == 0 ? 0 : (kind == 1 ? Cq : 2 * Cq)) + head * d + c0;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  if (act) {
+    const int col = chan_col(c, Cq, q_off, k_off, v_off);
+    const int s = token_seq[t];
+    const int q0 = qlocs[s], n = qlocs[s + 1] - q0;
+    const int start = seq_lens[s] - n;
+    const int jl = (int)t - q0;
+    const float* hist = conv_state + (long)state_slots[s] * (taps - 1) * C;
+    for (int back = 0; back < taps; ++back) {
+      float x[8];
+      if (jl - back >= 0) {
+        bf8_to_f32(*(const u16x8*)(proj + (t - back) * ld + col), x);
+      } else if (start > 0) {
+        const float* hp = hist + (long)(taps - 1 - back + jl) * C + c;
+        const f32x4 a = *(const f32x4*)hp, b = *(const f32x4*)(hp + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { x[e] = a[e]; x[e + 4] = b[e]; }
+      } else {
+        continue;  // before the start of the sequence: zeros
+      }
+      const float* wp = conv_wt + (long)(taps - 1 - back) * C + c;
+      const f32x4 w0 = *(const f32x4*)wp, w1 = *(const f32x4*)(wp + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        acc[e] += w0[e] * x[e];
+        acc[e + 4] += w1[e] * x[e + 4];
+      }
+    }
+  }
+  float ssq = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    acc[e] = acc[e] * sigmoid_f(acc[e]);
+    ssq += acc[e] * acc[e];
+  }
+#pragma unroll
+  for (int off = GS / 2; off > 0; off >>= 1) ssq += __shfl_xor(ssq, off, WAVE);
+  if (!act) return;
+  float f = 1.f;
+  if (kind != 2) {
+    f = 1.f / sqrtf(ssq + 1e-6f);
+    if (kind == 0) f *= 1.f / sqrtf((float)dk);
+  }
+  float* dst = (kind == 0 ? qn + (t * G + head) * (long)dk
+                          : (kind == 1 ? kn + (t * G + head) * (long)dk
+                                       : vv + (t * H + head) * (long)dv)) + c0;
+  f32x4 o0, o1;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) { o0[e] = acc[e] * f; o1[e] = acc[e + 4] * f; }
+  *(f32x4*)dst = o0;
+  *(f32x4*)(dst + 4) = o1;
 }
 
 // ---- low-rank gates ---------------------------------------------------------
@@ -113,17 +200,16 @@ __device__ __forceinline__ void low_rank_acc(
 #pragma unroll
     for (int r = 0; r < RMAX; ++r)
       w[r] = (col_ok && r0 + r < rank) ? w2t[(long)(r0 + r) * stride + col] : 0.f;
+    float x[GT];  // lane r holds input r of token tt
 #pragma unroll
-    for (int tt = 0; tt < GT; ++tt) {
-      const long t = t_base + tt;
-      if (t >= T) break;  // wave-uniform
-      const float x = (lane < RMAX && r0 + lane < rank)
-                          ? ldf<A>(in + t * ld + r0 + lane) : 0.f;
-      float a = 0.f;
+    for (int tt = 0; tt < GT; ++tt)
+      x[tt] = (t_base + tt < T && lane < RMAX && r0 + lane < rank)
+                  ? ldf<A>(in + (t_base + tt) * ld + r0 + lane) : 0.f;
+    // r outer, tokens inner: GT independent readlane + FMA chains
 #pragma unroll
-      for (int r = 0; r < RMAX; ++r) a += w[r] * lane_bcast(x, r);
-      acc[tt] += a;
-    }
+    for (int r = 0; r < RMAX; ++r)
+#pragma unroll
+      for (int tt = 0; tt < GT; ++tt) acc[tt] += w[r] * lane_bcast(x[tt], r);
   }
 }
 
@@ -374,18 +460,48 @@ __global__ void delta_out_kernel(A* __restrict__ out, long ldo, int out_off,
 extern "C" void mix_delta_prep(
     float* qn, float* kn, float* vv, float* decay, float* beta,
     const void* proj, long ld, int q_off, int k_off, int v_off, int b_off,
-    int a1_off, const float* conv_w, int taps, const float* a2, int rank,
+    int a1_off, const float* conv_w, const float* conv_wt, int taps,
+    const float* a2, int rank,
     const float* dt_bias, const float* a_log, float* conv_state,
     const int* state_slots, const int* qlocs, const int* seq_lens,
     const int* token_seq, long T, int S, int H, int G, int dk, int dv, int f32,
     hipStream_t s) {
-  const long units = T * (2 * G + H);
+  const long units = ((T + PT - 1) / PT) * (2 * G + H);
   const int grid = (int)((units + WPB - 1) / WPB);
   if (grid == 0) return;
   const dim3 ggrid((unsigned)((T + WPB * GT - 1) / (WPB * GT)), (unsigned)H);
   const int Cq = G * dk, C = 2 * Cq + H * dv;
   const long su = (long)S * C;
   const int sgrid = (int)((su + 255) / 256);
+  const int dmax = dk > dv ? dk : dv;
+  const int dm8 = (dmax + 7) / 8;
+  const bool vec = !f32 && conv_wt && dk % 8 == 0 && dv % 8 == 0 &&
+                   ld % 8 == 0 && q_off % 8 == 0 && k_off % 8 == 0 &&
+                   v_off % 8 == 0 && dm8 <= 32;
+  if (vec) {
+    const int GS = dm8 <= 4 ? 4 : (dm8 <= 8 ? 8 : (dm8 <= 16 ? 16 : 32));
+    const long tot = T * (2 * G + H);
+    const long waves = (tot + 64 / GS - 1) / (64 / GS);
+    const int vgrid = (int)((waves + WPB - 1) / WPB);
+#define LAUNCH_DV(GG)                                                          \
+  hipLaunchKernelGGL(delta_prep_vec_kernel<GG>, dim3(vgrid), dim3(WPB * WAVE), \
+                     0, s, qn, kn, vv, (const u16*)proj, ld, q_off, k_off,     \
+                     v_off, conv_wt, taps, conv_state, state_slots, qlocs,     \
+                     seq_lens, token_seq, T, H, G, dk, dv)
+    if (GS == 4) LAUNCH_DV(4);
+    else if (GS == 8) LAUNCH_DV(8);
+    else if (GS == 16) LAUNCH_DV(16);
+    else LAUNCH_DV(32);
+#undef LAUNCH_DV
+    hipLaunchKernelGGL(delta_gates_kernel<u16>, ggrid, dim3(WPB * WAVE), 0, s,
+                       decay, beta, (const u16*)proj, ld, b_off, a1_off, a2,
+                       rank, dt_bias, a_log, T, H, dk);
+    if (taps > 1)
+      hipLaunchKernelGGL(conv_state_update_kernel<u16>, dim3(sgrid), dim3(256),
+                         0, s, conv_state, (const u16*)proj, ld, q_off, k_off,
+                         v_off, taps, state_slots, qlocs, seq_lens, S, Cq, C);
+    return;
+  }
   if (f32) {
     hipLaunchKernelGGL(delta_prep_kernel<float>, dim3(grid), dim3(WPB * WAVE),
                        0, s, qn, kn, vv, (const float*)proj, ld, q_off, k_off,

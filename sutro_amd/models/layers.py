@@ -204,13 +204,15 @@ class GatedDeltaRule(nn.Module):
             # transposed copies of the low-rank up-projections, made once
             # (before any graph capture: capture is preceded by a warm-up run)
             self._t = (self.a2.detach().t().contiguous(),
-                       self.g2.detach().t().contiguous())
+                       self.g2.detach().t().contiguous(),
+                       self.conv_w.detach().t().contiguous())
         qn, kn, v, decay, beta = hops.delta_prep(
             proj, off[tag + "q"], off[tag + "k"], off[tag + "v"],
             off[tag + "b"], off[tag + "a1"], s.heads, s.kv_heads, s.dim,
             s.vdim, self.conv_w, self.a2, self.dt_bias, self.a_log,
             st.conv[self.layer_idx], fb.state_slots, fb.query_start_locs,
-            fb.seq_lens, token_seq=fb.token_seq, a2_t=self._t[0])
+            fb.seq_lens, token_seq=fb.token_seq, a2_t=self._t[0],
+            conv_w_t=self._t[2])
         o = hops.delta_scan(qn, kn, v, decay, beta, st.ssm[self.layer_idx],
                             fb.state_slots, fb.query_start_locs, fb.seq_lens)
         hops.delta_out(o, self.norm_w, proj, off[tag + "g1"], self.g2,

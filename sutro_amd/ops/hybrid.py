@@ -116,12 +116,16 @@ def local_attention(q, k_cache, v_cache, block_tables, seq_lens,
 
 def delta_prep(proj, q_off, k_off, v_off, b_off, a1_off, H, G, dk, dv,
                conv_w, a2, dt_bias, a_log, conv_state, state_slots,
-               query_start_locs, seq_lens, token_seq=None, a2_t=None):
-    """`a2_t`: a2 transposed and contiguous ([rank, H*dk], what the kernel
-    reads); made on the fly when the caller does not keep one."""
+               query_start_locs, seq_lens, token_seq=None, a2_t=None,
+               conv_w_t=None):
+    """`a2_t`, `conv_w_t`: a2 and conv_w transposed and contiguous ([rank,
+    H*dk] and [taps, C], what the kernels read); made on the fly when the
+    caller does not keep them."""
     if proj.is_cuda:
         if a2_t is None:
             a2_t = a2.t().contiguous()
+        if conv_w_t is None:
+            conv_w_t = conv_w.t().contiguous()
         T = proj.shape[0]
         f32 = dict(dtype=torch.float32, device=proj.device)
         qn = torch.empty((T, G, dk), **f32)
@@ -132,7 +136,7 @@ def delta_prep(proj, q_off, k_off, v_off, b_off, a1_off, H, G, dk, dv,
         _mix().delta_prep(qn, kn, v, decay, beta, proj, q_off, k_off, v_off,
                           b_off, a1_off, conv_w, a2_t, dt_bias, a_log,
                           conv_state, state_slots, query_start_locs, seq_lens,
-                          token_seq)
+                          token_seq, conv_w_t)
         return qn, kn, v, decay, beta
     return torch_ref.delta_prep(proj, q_off, k_off, v_off, b_off, a1_off, H,
                                 G, dk, dv, conv_w, a2, dt_bias, a_log,

@@ -195,6 +195,37 @@ def serve(host: str, port: int, device: str):
 
 
 @cli.command()
+@click.option("--model", required=True,
+              help="registry name, or a checkpoint directory holding "
+                   "config.json and *.safetensors (the model class is chosen "
+                   "by its config.json)")
+@click.option("--prompt", "prompts", multiple=True, required=True)
+@click.option("--max-tokens", default=64, show_default=True)
+@click.option("--temperature", default=0.8, show_default=True)
+@click.option("--device", default="auto", show_default=True)
+@click.option("--max-model-len", default=2048, show_default=True)
+def generate(model: str, prompts, max_tokens: int, temperature: float,
+             device: str, max_model_len: int):
+    """Generate locally with an in-process engine (no service, no job)."""
+    from .engine.engine import LLMEngine
+    from .engine.request import SamplingParams
+    from .service.models_map import resolve_engine_config
+
+    cfg = resolve_engine_config(model, device=device,
+                                max_model_len=max_model_len,
+                                max_num_seqs=max(8, len(prompts)))
+    if cfg.device.startswith("cuda"):
+        from .build import ensure_built
+
+        ensure_built(["_C", "_C_mix"] if cfg.spec.arch == "vodinex" else ["_C"])
+    eng = LLMEngine(cfg)
+    outs = eng.generate(list(prompts), sampling=SamplingParams(
+        max_tokens=max_tokens, temperature=temperature))
+    for p, o in zip(prompts, outs):
+        click.echo(json.dumps({"prompt": p, "output": o}))
+
+
+@cli.command()
 def docs():
     click.echo("see README.md and SURVEY.md in the repository")
 

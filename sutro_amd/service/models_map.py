@@ -39,7 +39,8 @@ def resolve_engine_config(
     spec = get_model_spec(model)
     if device == "auto":
         device = "cuda" if torch.cuda.is_available() else "cpu"
-    if device == "cpu" and spec.param_count() > _CPU_PARAM_LIMIT:
+    if (device == "cpu" and isinstance(spec, ModelSpec)
+            and spec.param_count() > _CPU_PARAM_LIMIT):
         spec = dev_proxy(spec)
     if (device.startswith("cuda") and spec.num_experts > 0
             and "max_num_seqs" not in kwargs):

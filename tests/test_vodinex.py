@@ -517,3 +517,48 @@ def test_greedy_generation_through_scheduler(tmp_path_factory, backend):
             assert tok == best or margin < 20 * limit(dtype), (n, tok, best)
             checked += 1
     assert checked >= 20
+
+
+def test_cli_generates_from_a_checkpoint_directory(tmp_path_factory):
+    """`sutro generate --model DIR`: the registry resolves the directory by
+    its config.json, the loader fills the model, the engine samples."""
+    import json
+
+    from click.testing import CliRunner
+
+    from sutro_amd.cli import cli
+
+    ck = checkpoint(tmp_path_factory, "config_a", config_a)
+    res = CliRunner().invoke(cli, ["generate", "--model", ck[0], "--prompt",
+                                   "hello there", "--prompt", "two",
+                                   "--max-tokens", "5", "--temperature", "0",
+                                   "--device", "cpu", "--max-model-len", "256"])
+    assert res.exit_code == 0, res.output
+    lines = [json.loads(x) for x in res.output.strip().splitlines()]
+    assert [x["prompt"] for x in lines] == ["hello there", "two"]
+
+
+def test_registry_resolves_architectures_by_config(tmp_path, tmp_path_factory):
+    import json
+
+    from sutro_amd.models.hybrid_spec import HybridSpec
+    from sutro_amd.models.registry import (ModelSpec, get_model_spec,
+                                           register_model_dir)
+
+    ck = checkpoint(tmp_path_factory, "config_b", config_b)
+    spec = get_model_spec(ck[0])
+    assert isinstance(spec, HybridSpec) and spec.arch == "vodinex"
+    assert spec.num_layers == 4 and spec.layers[0].mixer.conv == 1
+    assert spec.layers[1].mixer.right.decay_rank == 6      # from tensor shapes
+    assert register_model_dir("my-vodinex", ck[0]).name == "my-vodinex"
+    assert get_model_spec("my-vodinex").checkpoint_dir == ck[0]
+    (tmp_path / "config.json").write_text(json.dumps({
+        "architectures": ["Qwen3ForCausalLM"], "hidden_size": 64,
+        "num_hidden_layers": 2, "num_attention_heads": 4,
+        "num_key_value_heads": 2, "head_dim": 16, "intermediate_size": 128,
+        "vocab_size": 512}))
+    q = get_model_spec(str(tmp_path))
+    assert isinstance(q, ModelSpec) and q.num_kv_heads == 2
+    (tmp_path / "config.json").write_text(json.dumps({"architecture": "Nope"}))
+    with pytest.raises(KeyError):
+        get_model_spec(str(tmp_path))

@@ -29,6 +29,14 @@ def mix_available() -> bool:
 
 
 def _mix():
+    global _M, _M_ERR
+    if _M is None:  # the extension may have been built after this import
+        try:
+            import importlib
+
+            _M = importlib.import_module("sutro_amd._C_mix")
+        except Exception as e:
+            _M_ERR = f"{type(e).__name__}: {e}"
     if _M is None:
         raise RuntimeError(
             "sutro_amd HIP extension (_C_mix) is not built but a GPU tensor "

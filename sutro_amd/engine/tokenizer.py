@@ -212,11 +212,48 @@ def full_vocab_size() -> int:
     return BYTE_OFFSET + 256 + len(_load_merges())
 
 
-def get_tokenizer(vocab_size: Optional[int] = None) -> BPETokenizer:
+class IdTokenizer:
+    """Stand-in for models whose vocabulary is smaller than the byte
+    alphabet (fewer than 259 ids): there is no text mapping, prompts are
+    whitespace-separated token ids and outputs are printed the same way.
+    Token-id entry points (add_request, schedule replay) are unaffected."""
+
+    def __init__(self, vocab_size: int) -> None:
+        self.vocab_size = vocab_size
+
+    def encode(self, text: str, add_bos: bool = False) -> List[int]:
+        try:
+            ids = [int(x) for x in text.split()]
+        except ValueError:
+            raise ValueError(
+                f"this model's vocabulary ({self.vocab_size} ids) has no text "
+                f"mapping; pass whitespace-separated token ids") from None
+        if any(i < 0 or i >= self.vocab_size for i in ids):
+            raise ValueError("token id outside the vocabulary")
+        return ([BOS_ID] if add_bos and self.vocab_size > BOS_ID else []) + ids
+
+    def encode_batch(self, texts: List[str], add_bos: bool = False) -> List[List[int]]:
+        return [self.encode(t, add_bos) for t in texts]
+
+    def decode(self, ids: List[int]) -> str:
+        return " ".join(str(int(i)) for i in ids)
+
+    def render_prompt(self, user: str, system: Optional[str] = None) -> List[int]:
+        return self.encode(((system + " ") if system else "") + user,
+                           add_bos=True)
+
+    def render_prompts(self, users: List[str],
+                       system: Optional[str] = None) -> List[List[int]]:
+        return [self.render_prompt(u, system) for u in users]
+
+
+def get_tokenizer(vocab_size: Optional[int] = None):
     """The BPE tokenizer truncated to ``vocab_size`` (None = full). Cached
     per size; pass the model spec's vocab_size so sampled ids always fit the
     embedding table (model vocabs larger than the shipped tokenizer get the
     full tokenizer; the sampler masks the dead tail)."""
+    if vocab_size is not None and vocab_size < TOKENIZER_VOCAB:
+        return IdTokenizer(vocab_size)
     merges = _load_merges()
     full = BYTE_OFFSET + 256 + len(merges)
     v = full if vocab_size is None else min(vocab_size, full)

@@ -85,6 +85,20 @@ def config_b():
     ], eps=1e-6, mult=1.0)
 
 
+def config_c():
+    """A vocabulary smaller than the byte alphabet, widths that are not
+    multiples of 8 anywhere (merged projections and the merged output
+    projection need padding), head sizes of 6 and 10."""
+    return O.make_config(36, 50, [
+        O.parallel_layer(
+            O.attn_cfg(heads=3, kv_heads=1, dim=10, vdim=6, chunk=5,
+                       rot_dims=6, base=30.0, scale=0.4),
+            O.delta_cfg(heads=3, kv_heads=3, dim=6, vdim=10, conv=3),
+            0.9, 0.65, ff=20),
+        O.delta_layer(O.delta_cfg(heads=2, kv_heads=1, dim=10, vdim=6, conv=2)),
+    ], eps=2e-5, mult=0.8)
+
+
 _CACHE = {}
 
 
@@ -170,7 +184,7 @@ def check(ck, got, seqs, dtype, names=None):
 
 # ------------------------------------------------ whole prompts, decoding ---
 
-@pytest.mark.parametrize("cfg_fn", [config_a, config_b])
+@pytest.mark.parametrize("cfg_fn", [config_a, config_b, config_c])
 def test_whole_prompt(tmp_path_factory, backend, cfg_fn):
     ck = checkpoint(tmp_path_factory, cfg_fn.__name__, cfg_fn)
     eng = engine(ck, backend)
@@ -193,7 +207,7 @@ def test_first_tokens(tmp_path_factory, backend, cfg_fn):
     check(ck, got, seqs, backend[1], names=["n2", "n3"])
 
 
-@pytest.mark.parametrize("cfg_fn", [config_a, config_b])
+@pytest.mark.parametrize("cfg_fn", [config_a, config_b, config_c])
 def test_prefill_then_token_by_token(tmp_path_factory, backend, cfg_fn):
     ck = checkpoint(tmp_path_factory, cfg_fn.__name__, cfg_fn)
     eng = engine(ck, backend)

@@ -274,18 +274,39 @@ __global__ void conv_state_update_kernel(
   }
 }
 
-#define RPT 32  // state rows per lane
 #define TB 8    // tokens staged per step
 
+// sum over the R adjacent lanes of a column (R = 1, 2, 4, 8 or 16, aligned):
+// DPP moves inside the VALU, no LDS round trip. quad_perm covers the xor-1
+// and xor-2 steps; after them every lane of a quad holds the quad's sum, so
+// the mirror steps (lane i <- lane 7-i, then 15-i) complete rows of 8 and 16.
+template <int R>
+__device__ __forceinline__ float group_sum(float v) {
+  if (R >= 2)
+    v += __int_as_float(__builtin_amdgcn_update_dpp(
+        0, __float_as_int(v), 0xB1, 0xF, 0xF, true));   // quad_perm 1,0,3,2
+  if (R >= 4)
+    v += __int_as_float(__builtin_amdgcn_update_dpp(
+        0, __float_as_int(v), 0x4E, 0xF, 0xF, true));   // quad_perm 2,3,0,1
+  if (R >= 8)
+    v += __int_as_float(__builtin_amdgcn_update_dpp(
+        0, __float_as_int(v), 0x141, 0xF, 0xF, true));  // row_half_mirror
+  if (R >= 16)
+    v += __int_as_float(__builtin_amdgcn_update_dpp(
+        0, __float_as_int(v), 0x140, 0xF, 0xF, true));  // row_mirror
+  return v;
+}
+
 // Token-by-token scan. Block = (sequence, head, group of 256/R columns);
-// lane (col, r) keeps rows {((n/4)*R + r)*4 + n%4 : n < 32} of its column of
-// S in registers (rows past dk stay zero: their k and q are staged as 0 and
+// lane (col, r) keeps rows {((n/4)*R + r)*4 + n%4 : n < RPT} of its column of
+// S in registers (RPT = 32, or 16 to double the number of waves when a
+// launch would leave SIMDs idle) (rows past dk stay zero: their k and q are staged as 0 and
 // their decay as 1). k, q, decay, v and beta of TB tokens at a time are
 // staged through a double-buffered LDS tile: the global loads of tile s+1
 // are issued before the arithmetic of tile s and parked in registers. With
 // this row mapping the R lanes of a column read consecutive float4s of a
 // staged row, and all columns read the same addresses (LDS broadcast).
-template <int R>
+template <int R, int RPT>
 __global__ void __launch_bounds__(256) delta_scan_kernel(
     float* __restrict__ o, const float* __restrict__ qn,
     const float* __restrict__ kn, const float* __restrict__ vv,
@@ -380,9 +401,7 @@ __global__ void __launch_bounds__(256) delta_scan_kernel(
           dot += S[m * 4 + j] * k4[j];
         }
       }
-#pragma unroll
-      for (int off = R >> 1; off > 0; off >>= 1)
-        dot += __shfl_xor(dot, off, WAVE);
+      dot = group_sum<R>(dot);
       const float uu = bt * (vt - dot);
       float out = 0.f;
 #pragma unroll
@@ -394,9 +413,7 @@ __global__ void __launch_bounds__(256) delta_scan_kernel(
           out += S[m * 4 + j] * q4[j];
         }
       }
-#pragma unroll
-      for (int off = R >> 1; off > 0; off >>= 1)
-        out += __shfl_xor(out, off, WAVE);
+      out = group_sum<R>(out);
       if (r == 0 && cv) o[((long)(t0 + tok) * H + h) * dv + col] = out;
     }
   }
@@ -537,19 +554,36 @@ extern "C" void mix_delta_scan(float* o, const float* qn, const float* kn,
                                const int* seq_lens, int S, int H, int G, int dk,
                                int dv, hipStream_t s) {
   int R = 1;
-  while (R * RPT < dk) R <<= 1;  // dk <= 256 -> R <= 8
+  while (R * 32 < dk) R <<= 1;  // dk <= 256 -> R <= 8 at 32 rows a lane
+  int rpt = 32;
+  {
+    // few sequences x heads: 16 rows a lane doubles the waves in flight
+    const long blocks32 = (long)S * H * ((dv + 256 / R - 1) / (256 / R));
+    if (blocks32 < 512 && dk > 16) {
+      rpt = 16;
+      R = 2;
+      while (R * 16 < dk) R <<= 1;  // R <= 16
+    }
+  }
   const int cols_pb = 256 / R;
   const int col_groups = (dv + cols_pb - 1) / cols_pb;
   const long grid = (long)S * H * col_groups;
   if (grid == 0) return;
-#define LAUNCH_SCAN(RR)                                                     \
-  hipLaunchKernelGGL(delta_scan_kernel<RR>, dim3((unsigned)grid), dim3(256), \
-                     0, s, o, qn, kn, vv, decay, beta, ssm, state_slots,     \
-                     qlocs, seq_lens, H, G, dk, dv, col_groups)
-  if (R == 1) LAUNCH_SCAN(1);
-  else if (R == 2) LAUNCH_SCAN(2);
-  else if (R == 4) LAUNCH_SCAN(4);
-  else LAUNCH_SCAN(8);
+#define LAUNCH_SCAN(RR, PP)                                                  \
+  hipLaunchKernelGGL((delta_scan_kernel<RR, PP>), dim3((unsigned)grid),      \
+                     dim3(256), 0, s, o, qn, kn, vv, decay, beta, ssm,       \
+                     state_slots, qlocs, seq_lens, H, G, dk, dv, col_groups)
+  if (rpt == 32) {
+    if (R == 1) LAUNCH_SCAN(1, 32);
+    else if (R == 2) LAUNCH_SCAN(2, 32);
+    else if (R == 4) LAUNCH_SCAN(4, 32);
+    else LAUNCH_SCAN(8, 32);
+  } else {
+    if (R == 2) LAUNCH_SCAN(2, 16);
+    else if (R == 4) LAUNCH_SCAN(4, 16);
+    else if (R == 8) LAUNCH_SCAN(8, 16);
+    else LAUNCH_SCAN(16, 16);
+  }
 #undef LAUNCH_SCAN
 }
 

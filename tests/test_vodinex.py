@@ -216,11 +216,13 @@ def test_prefill_then_token_by_token(tmp_path_factory, backend, cfg_fn):
     check(ck, got, seqs, backend[1])
 
 
-def test_portions_of_many_sizes(tmp_path_factory, backend):
+@pytest.mark.parametrize("page", [8, 32])
+def test_portions_of_many_sizes(tmp_path_factory, backend, page):
     """Prompt pieces of 2, 3, 1, 11, 2, 5 ... tokens: cuts inside pages,
-    inside chunks and inside the filters' reach."""
+    inside chunks and inside the filters' reach. With pages of 32 the bf16
+    prompt pieces take the matrix-core attention kernel."""
     ck = checkpoint(tmp_path_factory, "config_a", config_a)
-    eng = engine(ck, backend)
+    eng = engine(ck, backend, page=page, blocks=24)
     seqs = {"s": tokens_for(ck[1], 62, 2)}
     sizes = [2, 3, 1, 11, 2, 5, 1, 1, 13, 2, 8, 7, 2, 4]
     assert sum(sizes) == 62
@@ -240,11 +242,12 @@ def test_long_decoding(tmp_path_factory, backend):
 
 # ----------------------------------------------------- batches, reuse -------
 
-def test_mixed_batch_equals_each_alone(tmp_path_factory, backend):
+@pytest.mark.parametrize("page", [8, 32])
+def test_mixed_batch_equals_each_alone(tmp_path_factory, backend, page):
     """Unequal requests in one batch (prompt pieces beside single tokens,
     requests that sit out a step) give what each gives alone."""
     ck = checkpoint(tmp_path_factory, "config_a", config_a)
-    eng = engine(ck, backend)
+    eng = engine(ck, backend, page=page, blocks=24)
     seqs = {"a": tokens_for(ck[1], 40, 4), "b": tokens_for(ck[1], 17, 5),
             "c": tokens_for(ck[1], 9, 6), "d": tokens_for(ck[1], 26, 7)}
     schedule = [

@@ -1,8 +1,9 @@
 // Gated delta rule with one decay per head and key channel.
 //
 //   delta_prep         short causal depthwise filter + silu on the q|k|v
-//                      channels, unit-norm q (times dk^-1/2) and k, beta =
-//                      sigmoid, decay = exp(-exp(A_log) * softplus(a2 a1 + dt))
+//                      channels, unit-norm q (times dk^-1/2) and k
+//   delta_gates        beta = sigmoid, decay = exp(-exp(A_log) *
+//                      softplus(a2 a1 + dt_bias)) per head and key channel
 //   conv_state_update  keeps the last taps-1 raw filter inputs per sequence
 //   delta_scan         S <- decay * S; u = beta (v - S^T k); S <- S + k u^T;
 //                      o = S^T q, token by token, S [dk, dv] fp32 per head
@@ -15,8 +16,9 @@
 //
 // delta_scan maps the state onto lanes by COLUMN: the dv columns of S never
 // interact, so a column is owned by R adjacent lanes holding dk/R rows each
-// in registers; one token costs two R-lane shuffle reductions and no LDS
-// traffic or barriers. Blocks cover (sequence, head, group of columns).
+// in registers; one token costs two R-lane sums (DPP moves) and broadcast
+// reads of the staged k, q and decay rows. Blocks cover (sequence, head,
+// group of columns).
 #include "mix_common.h"
 
 #define WPB 4

@@ -579,3 +579,13 @@ def test_registry_resolves_architectures_by_config(tmp_path, tmp_path_factory):
     (tmp_path / "config.json").write_text(json.dumps({"architecture": "Nope"}))
     with pytest.raises(KeyError):
         get_model_spec(str(tmp_path))
+
+
+def test_service_job_on_a_checkpoint_directory(tmp_path_factory, local_client):
+    """A checkpoint directory is a model name for the job service too."""
+    ck = checkpoint(tmp_path_factory, "config_a", config_a)
+    job = local_client.infer(["alpha", "beta gamma"], model=ck[0],
+                             sampling_params={"max_tokens": 4, "temperature": 0},
+                             stay_attached=False)
+    out = local_client.await_job_completion(job, timeout=120)
+    assert out is not None and len(out) == 2

@@ -35,14 +35,17 @@ def limit(dtype):
     return 2e-4 if dtype == torch.float32 else 6e-2
 
 
-def rel_err(got, want):
-    """Root mean square of the difference (mean over the vocabulary taken
-    off), relative to the spread of the expected logits; worst row."""
+def row_errors(got, want):
+    """Per position: root mean square of the difference (mean over the
+    vocabulary taken off), relative to the spread of the expected logits."""
     d = got.double().cpu() - want
     d = d - d.mean(-1, keepdim=True)
     ref = want - want.mean(-1, keepdim=True)
-    return float((d.pow(2).mean(-1).sqrt()
-                  / ref.pow(2).mean().sqrt()).max())
+    return d.pow(2).mean(-1).sqrt() / ref.pow(2).mean().sqrt()
+
+
+def rel_err(got, want):
+    return float(row_errors(got, want).max())
 
 
 # ------------------------------------------------------------- configs ------
@@ -170,16 +173,15 @@ def check(ck, got, seqs, dtype, names=None):
     for name in names or got:
         want = oracle_logits(ck, seqs[name])
         assert got[name].shape == want.shape
+        rows = row_errors(got[name], want)
         if dtype == torch.float32:
-            e = rel_err(got[name], want)
-            assert e < limit(dtype), f"{name}: relative error {e}"
+            assert float(rows.max()) < limit(dtype), \
+                f"{name}: relative error {float(rows.max())}"
         else:
-            rows = [rel_err(got[name][i:i + 1], want[i:i + 1]) *
-                    float((want[i] - want[i].mean()).pow(2).mean().sqrt()
-                          / (want - want.mean(-1, keepdim=True)).pow(2).mean().sqrt())
-                    for i in range(want.shape[0])]
-            assert sum(rows) / len(rows) < limit(dtype), f"{name}: mean {rows}"
-            assert max(rows) < 5 * limit(dtype), f"{name}: worst {max(rows)}"
+            assert float(rows.mean()) < limit(dtype), \
+                f"{name}: mean relative error {float(rows.mean())}"
+            assert float(rows.max()) < 5 * limit(dtype), \
+                f"{name}: worst relative error {float(rows.max())}"
 
 
 # ------------------------------------------------ whole prompts, decoding ---

@@ -48,5 +48,8 @@ class ForwardBatch:
     # models with per-sequence recurrent state / per-token sequence lookups
     state_slots: Optional[torch.Tensor] = None  # [S] int32 state slot per seq
     token_seq: Optional[torch.Tensor] = None    # [T] int32 seq index per row
+    # [T] long: the token before each row's token in its sequence, -1 for a
+    # sequence's first token (models whose embedding looks at token pairs)
+    prev_ids: Optional[torch.Tensor] = None
     # per-step scratch shared by a model's layers (e.g. rotation tables)
     aux: dict = field(default_factory=dict)

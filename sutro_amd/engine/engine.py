@@ -258,6 +258,8 @@ class LLMEngine:
         input_ids = np.empty(T, dtype=np.int64)
         positions = np.empty(T, dtype=np.int64)
         slots = np.empty(T, dtype=np.int64)
+        want_prev = getattr(self.model, "uses_prev_ids", False)
+        prev_ids = np.full(T, -1, dtype=np.int64) if want_prev else None
         qlocs = np.zeros(S + 1, dtype=np.int32)
         seq_lens = np.empty(S, dtype=np.int32)
         bs = self.kv.block_size
@@ -275,6 +277,9 @@ class LLMEngine:
                                      if pos < req.total_len else 0)
                 positions[cursor] = pos
                 slots[cursor] = table[pos // bs] * bs + pos % bs
+                if want_prev and pos > 0:
+                    prev_ids[cursor] = (input_ids[cursor - 1] if j > 0
+                                        else req.token_at(pos - 1))
                 cursor += 1
             qlocs[s + 1] = cursor
             seq_lens[s] = start + c
@@ -314,6 +319,8 @@ class LLMEngine:
         return ForwardBatch(
             state_slots=state_slots,
             token_seq=token_seq,
+            prev_ids=(torch.from_numpy(prev_ids).to(dev) if want_prev
+                      else None),
             input_ids=torch.from_numpy(input_ids).to(dev),
             positions=torch.from_numpy(positions).to(dev),
             slot_mapping=torch.from_numpy(slots).to(dev),

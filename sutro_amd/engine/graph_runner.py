@@ -54,6 +54,11 @@ class DecodeGraphRunner:
         self.has_state = engine.kv.state is not None
         self.d_state = torch.zeros(B, dtype=torch.int32, device=dev)
         self.h_state = torch.zeros(B, dtype=torch.int32, pin_memory=True)
+        # models whose embedding looks at token pairs: the token before each
+        # row's token (-1 = none; padding rows)
+        self.has_prev = getattr(engine.model, "uses_prev_ids", False)
+        self.d_prev = torch.full((B,), -1, dtype=torch.long, device=dev)
+        self.h_prev = torch.full((B,), -1, dtype=torch.long, pin_memory=True)
         # pinned host staging
         self.h_ids = torch.zeros(B, dtype=torch.long, pin_memory=True)
         self.h_pos = torch.zeros(B, dtype=torch.long, pin_memory=True)
@@ -95,6 +100,7 @@ class DecodeGraphRunner:
             prefill_token_count=0,
             state_slots=self.d_state[:n] if self.has_state else None,
             token_seq=self.d_qlocs[:n],
+            prev_ids=self.d_prev[:n] if self.has_prev else None,
         )
 
     @torch.no_grad()
@@ -142,6 +148,11 @@ class DecodeGraphRunner:
         if self.has_state:
             self.d_state[:bucket].copy_(self.h_state[:bucket],
                                         non_blocking=True)
+        if self.has_prev:
+            # with lagged ids (async decode) the host-staged ids ARE the
+            # tokens before the overriding ones
+            src = self.h_ids if ids_override is not None else self.h_prev
+            self.d_prev[:bucket].copy_(src[:bucket], non_blocking=True)
         if ids_override is not None:
             self.d_ids[:n].copy_(ids_override, non_blocking=True)
         if self._h2d_done is not None:
@@ -200,6 +211,13 @@ class DecodeGraphRunner:
             st[:n] = np.fromiter((slots_of[r.req_id] for r in sb.reqs),
                                  np.int32, n)
             st[n:bucket] = kv.state.scratch_slot
+        if getattr(self, "has_prev", False):
+            pv = self.h_prev.numpy()
+            pv[:n] = np.fromiter(
+                ((r.token_at(r.num_computed_tokens - 1)
+                  if r.num_computed_tokens > 0 else -1) for r in sb.reqs),
+                np.int64, n)
+            pv[n:bucket] = -1
         if n < bucket:  # padding rows target the reserved scratch block
             ids[n:bucket] = 0
             pos[n:bucket] = 0

@@ -44,21 +44,28 @@ class RecurrentStateCache:
         conv[i]  [slots, taps-1, channels] fp32 — the last taps-1 inputs of the
                  layer's short filters, oldest first;
         ssm[i]   [slots, heads, dk, dv] fp32 — the delta-rule memory.
+    A layer may instead describe its state as a dict name -> per-slot shape;
+    it then gets fp32 tensors named[i][name] of shape [slots, *shape] (the
+    mLSTM keeps its matrix memory and its stabiliser this way).
     A slot is not cleared when it is handed out again: the kernels start from
     zero whenever a sequence's first token (position 0) is in the batch.
     Slot 0 is reserved as scratch for padded graph rows."""
 
-    def __init__(self, num_slots: int,
-                 shapes: Sequence[Optional[Tuple[int, int, int, int, int]]],
-                 device: str) -> None:
+    def __init__(self, num_slots: int, shapes: Sequence, device: str) -> None:
         self.num_slots = num_slots + 1
         self.conv: List[Optional[torch.Tensor]] = []
         self.ssm: List[Optional[torch.Tensor]] = []
+        self.named: List[Optional[Dict[str, torch.Tensor]]] = []
         for sh in shapes:
-            if sh is None:
+            if sh is None or isinstance(sh, dict):
                 self.conv.append(None)
                 self.ssm.append(None)
+                self.named.append(None if sh is None else {
+                    k: torch.zeros((self.num_slots,) + tuple(v),
+                                   dtype=torch.float32, device=device)
+                    for k, v in sh.items()})
                 continue
+            self.named.append(None)
             ch, taps, heads, dk, dv = sh
             self.conv.append(torch.zeros(self.num_slots, max(1, taps - 1), ch,
                                          dtype=torch.float32, device=device))

@@ -64,7 +64,60 @@ class ParallelMixerSpec:
     right_scale: float
 
 
-MixerSpec = Union[AttnMixerSpec, DeltaMixerSpec, ParallelMixerSpec]
+@dataclass(frozen=True)
+class TiedAttnMixerSpec:
+    """Windowed softmax attention whose values are its raw keys (no value
+    projection): q and k are RMS-normed over the whole projection (all heads
+    at once), q is scaled by 1 + temp_coef * ln(floor((p+1)/temp_every) + 1)
+    at position p (temp_every 0 = off), and with `dist_bias` the score of
+    query i and key j is lowered by r1[h] * ln(1 + r2[h] * (i - j)). No
+    rotation. ``window``: a query sees itself and the window-1 keys before it
+    (0 = unlimited)."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    scale: float
+    window: int = 0
+    temp_coef: float = 0.0
+    temp_every: int = 0
+    dist_bias: bool = True
+
+
+@dataclass(frozen=True)
+class LatentAttnMixerSpec:
+    """Attention through low-rank latents, without positions: queries are
+    up-projected from a normed latent of size q_rank; keys and values are
+    up-projected per head from one normed latent of size kv_rank, which is all
+    the cache holds. The concatenated heads pass an elementwise sigmoid gate.
+    ``kv_from``: index of an earlier layer whose cached latent this layer
+    reads instead of making its own."""
+
+    heads: int
+    dim: int
+    vdim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    window: int = 0
+    kv_from: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class MLSTMMixerSpec:
+    """mLSTM matrix memory: per head a [dim, vdim] state with exponential
+    input gate, sigmoid forget gate (both soft-capped at ``gate_cap`` in log
+    space) and a running-maximum stabiliser; read-out normed per head and
+    gated elementwise."""
+
+    heads: int
+    dim: int
+    vdim: int
+    gate_cap: float
+
+
+MixerSpec = Union[AttnMixerSpec, DeltaMixerSpec, ParallelMixerSpec,
+                  TiedAttnMixerSpec, LatentAttnMixerSpec, MLSTMMixerSpec]
 
 
 @dataclass(frozen=True)
@@ -89,6 +142,11 @@ class HybridSpec:
     residual_mult: float = 1.0
     max_context: int = 32768
     checkpoint_dir: Optional[str] = None
+    # hashed bigram table added to the token embedding: (buckets, multiplier
+    # of the previous token, multiplier of the current token); None = none
+    bigram: Optional[Tuple[int, int, int]] = None
+    pos_base: float = 0.0        # base of the additive sinusoid (0 = none)
+    logit_scale: float = 1.0
     # behavior flags shared with ModelSpec
     reasoning: bool = False
     embedding: bool = False
@@ -115,6 +173,8 @@ class HybridSpec:
             return h * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)
                         + m.heads) + m.heads * m.vdim * h
 
+        if self.arch == "ruludra":
+            return self._sandwich_param_count()
         for layer in self.layers:
             m = layer.mixer
             if isinstance(m, ParallelMixerSpec):
@@ -126,6 +186,31 @@ class HybridSpec:
             n += h * h                      # residual gate of the mixer
             if layer.ff:
                 n += 3 * h * layer.ff + h * h
+        return n
+
+    def _sandwich_param_count(self) -> int:
+        h = self.hidden_size
+        n = 2 * self.vocab_size * h + h
+        if self.bigram:
+            n += (self.bigram[0] + 1) * h
+        for i, layer in enumerate(self.layers):
+            m = layer.mixer
+            if isinstance(m, TiedAttnMixerSpec):
+                qd, kd = m.heads * m.dim, m.kv_heads * m.dim
+                n += h * (qd + kd) + qd + kd + 2 * m.heads + qd * h
+            elif isinstance(m, LatentAttnMixerSpec):
+                hv = m.heads * m.vdim
+                n += h * m.q_rank + m.q_rank + m.heads * m.dim * m.q_rank
+                if m.kv_from is None:
+                    n += h * m.kv_rank + m.kv_rank
+                n += (m.heads * m.dim + hv) * m.kv_rank + 2 * hv * h
+            elif isinstance(m, MLSTMMixerSpec):
+                hv = m.heads * m.vdim
+                n += h * (2 * m.heads * m.dim + 2 * hv + 2 * m.heads)
+                n += 2 * m.heads + hv + hv * h
+            n += 2 * h + (i + 2)
+            if layer.ff:
+                n += 2 * h * layer.ff + 4 + 2 * h
         return n
 
     def active_param_count(self) -> int:
@@ -196,3 +281,71 @@ def vodinex_spec(config: dict, name: str = "vodinex",
                       residual_mult=float(config["residual_mult"]),
                       max_context=int(config.get("max_context", 1 << 20)),
                       checkpoint_dir=checkpoint_dir)
+
+
+def ruludra_spec(config: dict, name: str = "ruludra",
+                 checkpoint_dir: Optional[str] = None,
+                 tensor_shapes: Optional[dict] = None) -> HybridSpec:
+    """Build the spec of a Ruludra checkpoint from its ``config.json``: a
+    list of layers, each with a tied-value windowed attention, a latent
+    attention or an mLSTM mixer and an optional PolyNorm feed-forward; token +
+    hashed-bigram + sinusoid embedding; every layer's input is a learned
+    weighted sum of the embedding output and all earlier layer results.
+    A latent's query rank is `q_rank` of the mixer dict, or else the row count
+    of ``<mixer>.dq`` in ``tensor_shapes``."""
+    shapes = tensor_shapes or {}
+    layers = []
+    for i, lc in enumerate(config["layers"]):
+        kind = lc["type"]
+        m = lc["mixer"]
+        mask = m.get("mask") or {}
+        if kind == "attention":
+            if int(m.get("vdim", m["dim"])) != int(m["dim"]):
+                raise ValueError(f"layer {i}: values are the keys, so vdim "
+                                 f"must equal dim")
+            qt = m.get("q_temp") or {}
+            mixer: MixerSpec = TiedAttnMixerSpec(
+                heads=int(m["heads"]), kv_heads=int(m["kv_heads"]),
+                dim=int(m["dim"]), scale=float(m["scale"]),
+                window=int(mask.get("size", 0)),
+                temp_coef=float(qt.get("coef", 0.0)),
+                temp_every=int(qt.get("every", 0)))
+        elif kind == "latent_attention":
+            src = m.get("kv_from")
+            dq = shapes.get(f"l{i}.mix.dq")
+            if src is not None:
+                src = int(src)
+                other = config["layers"][src] if 0 <= src < i else None
+                if (other is None or other["type"] != "latent_attention"
+                        or other["mixer"].get("kv_from") is not None
+                        or int(other["mixer"]["kv_rank"]) != int(m["kv_rank"])):
+                    raise ValueError(
+                        f"layer {i}: kv_from must name an earlier latent "
+                        f"layer of equal kv_rank that owns its latent")
+            mixer = LatentAttnMixerSpec(
+                heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                q_rank=int(m["q_rank"]) if "q_rank" in m else int(dq[0]),
+                kv_rank=int(m["kv_rank"]), scale=float(m["scale"]),
+                window=int(mask.get("size", 0)), kv_from=src)
+        elif kind == "mlstm":
+            mixer = MLSTMMixerSpec(heads=int(m["heads"]), dim=int(m["dim"]),
+                                   vdim=int(m["vdim"]),
+                                   gate_cap=float(m["gate_cap"]))
+        else:
+            raise ValueError(f"unknown layer type {kind!r} in layer {i}")
+        mlp = lc.get("mlp")
+        if mlp is not None and mlp.get("kind", "dense") != "dense":
+            raise ValueError(f"unknown feed-forward kind {mlp['kind']!r}")
+        layers.append(HybridLayerSpec(kind=kind, mixer=mixer,
+                                      ff=int(mlp["ff"]) if mlp else 0,
+                                      ff_kind="poly_norm"))
+    big = (config.get("embedding") or {}).get("bigram")
+    return HybridSpec(
+        name=name, arch="ruludra", hidden_size=int(config["width"]),
+        vocab_size=int(config["vocab"]), layers=tuple(layers),
+        norm_eps=float(config["norm"]["eps"]),
+        max_context=int(config.get("max_context", 1 << 20)),
+        checkpoint_dir=checkpoint_dir,
+        bigram=(int(big["buckets"]), int(big["mul_prev"]),
+                int(big["mul_cur"])) if big else None,
+        pos_base=10000.0, logit_scale=float(config.get("logit_scale", 1.0)))

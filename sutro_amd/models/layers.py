@@ -18,7 +18,8 @@ import torch.nn.functional as F
 from ..engine.batch import ForwardBatch
 from ..engine.kv_cache import PagedKVCache
 from ..ops import hybrid as hops
-from .hybrid_spec import AttnMixerSpec, DeltaMixerSpec
+from .hybrid_spec import (AttnMixerSpec, DeltaMixerSpec, LatentAttnMixerSpec,
+                          MLSTMMixerSpec, TiedAttnMixerSpec)
 
 _ALIGN = 8  # section starts are multiples of 8 columns (16 B in bf16)
 
@@ -217,3 +218,222 @@ class GatedDeltaRule(nn.Module):
                             fb.state_slots, fb.query_start_locs, fb.seq_lens)
         hops.delta_out(o, self.norm_w, proj, off[tag + "g1"], self.g2,
                        self.eps, out, out_off, out_scale, g2_t=self._t[1])
+
+
+class TiedWindowAttention(nn.Module):
+    """Windowed grouped-query attention whose values are its raw keys: whole-
+    projection q/k RMS norm, position-dependent query temperature, logarithmic
+    distance bias per head, no rotation and no value projection. Works on the
+    q and k sections of the sublayer's merged projection."""
+
+    def __init__(self, spec: TiedAttnMixerSpec, eps: float, layer_idx: int):
+        super().__init__()
+        self.spec = spec
+        self.eps = eps
+        self.layer_idx = layer_idx
+        if spec.heads % spec.kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+        f32 = torch.float32
+        self.q_norm = nn.Parameter(torch.ones(spec.heads * spec.dim, dtype=f32))
+        self.k_norm = nn.Parameter(torch.ones(spec.kv_heads * spec.dim, dtype=f32))
+        if spec.dist_bias:
+            self.r1 = nn.Parameter(torch.zeros(spec.heads, dtype=f32))
+            self.r2 = nn.Parameter(torch.zeros(spec.heads, dtype=f32))
+
+    def in_sections(self, tag: str):
+        s = self.spec
+        return [(tag + "q", s.heads * s.dim, False),
+                (tag + "k", s.kv_heads * s.dim, False)]
+
+    @property
+    def out_width(self) -> int:
+        return self.spec.heads * self.spec.dim
+
+    def kv_shape(self):
+        return (self.spec.kv_heads, self.spec.dim, self.spec.dim)
+
+    def state_shape(self):
+        return None
+
+    def param_targets(self, prefix: str, ck: str):
+        s = self.spec
+        t = {ck + ".q.norm": (prefix + "q_norm", 0, 0, s.heads * s.dim, 1.0),
+             ck + ".k.norm": (prefix + "k_norm", 0, 0, s.kv_heads * s.dim, 1.0)}
+        if s.dist_bias:
+            t[ck + ".r1"] = (prefix + "r1", 0, 0, s.heads, 1.0)
+            t[ck + ".r2"] = (prefix + "r2", 0, 0, s.heads, 1.0)
+        return t
+
+    def section_names(self, tag: str, ck: str):
+        return {tag + "q": ck + ".q", tag + "k": ck + ".k"}
+
+    def forward(self, proj: torch.Tensor, off: Dict[str, int], tag: str,
+                fb: ForwardBatch, kv: PagedKVCache, out: torch.Tensor,
+                out_off: int, out_scale: float) -> None:
+        s = self.spec
+        kc, vc = kv.k_cache[self.layer_idx], kv.v_cache[self.layer_idx]
+        q = hops.tied_attn_prep(
+            proj, off[tag + "q"], off[tag + "k"], s.heads, s.kv_heads, s.dim,
+            self.q_norm, self.k_norm, self.eps, fb.positions, s.temp_coef,
+            s.temp_every, fb.slot_mapping, kc, vc)
+        hops.local_attention(
+            q, kc, vc, fb.block_tables, fb.seq_lens, fb.query_start_locs,
+            s.scale, 0, s.window, proj, -1, out, out_off, out_scale,
+            token_seq=fb.token_seq, tile_seq=fb.tile_seq, tile_q0=fb.tile_q0,
+            prefill_rows=fb.prefill_token_count,
+            bias_r1=self.r1 if s.dist_bias else None,
+            bias_r2=self.r2 if s.dist_bias else None)
+
+
+class LatentAttention(nn.Module):
+    """Attention through low-rank latents without positions. The cache holds
+    only the normed key/value latent c [kv_rank] of every token (one "head" of
+    a paged K cache; no V pages). Attention runs in latent space: with per-head
+    up-projections K_h = U^k_h c and V_h = U^v_h c,
+        score = q_h . (U^k_h c) = ((U^k_h)^T q_h) . c,
+        out_h = U^v_h (sum_j p_j c_j),
+    so queries are folded through U^k once per token, one shared latent serves
+    all heads as key and value, and U^v is applied to the attended latent. A
+    layer with `kv_from` reads another layer's latent pages and writes none."""
+
+    def __init__(self, spec: LatentAttnMixerSpec, eps: float, layer_idx: int,
+                 dtype: torch.dtype):
+        super().__init__()
+        self.spec = spec
+        self.eps = eps
+        self.layer_idx = layer_idx
+        s = spec
+        f32 = torch.float32
+        self.dq_norm = nn.Parameter(torch.ones(s.q_rank, dtype=f32))
+        if s.kv_from is None:
+            self.dkv_norm = nn.Parameter(torch.ones(s.kv_rank, dtype=f32))
+        self.uq = nn.Parameter(torch.zeros(s.heads * s.dim, s.q_rank, dtype=dtype))
+        self.uk = nn.Parameter(torch.zeros(s.heads * s.dim, s.kv_rank, dtype=dtype))
+        self.uv = nn.Parameter(torch.zeros(s.heads * s.vdim, s.kv_rank, dtype=dtype))
+
+    def in_sections(self, tag: str):
+        s = self.spec
+        secs = [(tag + "dq", s.q_rank, False)]
+        if s.kv_from is None:
+            secs.append((tag + "dkv", s.kv_rank, False))
+        secs.append((tag + "g", s.heads * s.vdim, False))
+        return secs
+
+    @property
+    def out_width(self) -> int:
+        return self.spec.heads * self.spec.vdim
+
+    def kv_shape(self):
+        # one latent "head" as keys; values are read from the same pages
+        return (1, self.spec.kv_rank, 0) if self.spec.kv_from is None else None
+
+    def state_shape(self):
+        return None
+
+    def param_targets(self, prefix: str, ck: str):
+        s = self.spec
+        t = {ck + ".dq.norm": (prefix + "dq_norm", 0, 0, s.q_rank, 1.0),
+             ck + ".uq": (prefix + "uq", 0, 0, s.heads * s.dim, 1.0),
+             ck + ".uk": (prefix + "uk", 0, 0, s.heads * s.dim, 1.0),
+             ck + ".uv": (prefix + "uv", 0, 0, s.heads * s.vdim, 1.0)}
+        if s.kv_from is None:
+            t[ck + ".dkv.norm"] = (prefix + "dkv_norm", 0, 0, s.kv_rank, 1.0)
+        return t
+
+    def section_names(self, tag: str, ck: str):
+        n = {tag + "dq": ck + ".dq", tag + "g": ck + ".g"}
+        if self.spec.kv_from is None:
+            n[tag + "dkv"] = ck + ".dkv"
+        return n
+
+    def forward(self, proj: torch.Tensor, off: Dict[str, int], tag: str,
+                fb: ForwardBatch, kv: PagedKVCache, out: torch.Tensor,
+                out_off: int, out_scale: float) -> None:
+        s = self.spec
+        T = proj.shape[0]
+        H, dk, dv, R = s.heads, s.dim, s.vdim, s.kv_rank
+        dev, dt = proj.device, proj.dtype
+        cq = torch.empty((T, s.q_rank), dtype=dt, device=dev)
+        hops.section_rmsnorm(proj, off[tag + "dq"], s.q_rank, self.dq_norm,
+                             self.eps, cq)
+        src = self.layer_idx if s.kv_from is None else s.kv_from
+        cache = kv.k_cache[src]                    # [blocks, 1, page, R]
+        if s.kv_from is None:
+            hops.section_rmsnorm(proj, off[tag + "dkv"], R, self.dkv_norm,
+                                 self.eps, cache.view(-1, R),
+                                 rows=fb.slot_mapping)
+        q = F.linear(cq, self.uq)                  # [T, H*dk]
+        qa = torch.empty((T, H, R), dtype=dt, device=dev)
+        torch.bmm(q.view(T, H, dk).transpose(0, 1), self.uk.view(H, dk, R),
+                  out=qa.transpose(0, 1))
+        lat = torch.empty((T, H * R), dtype=dt, device=dev)
+        hops.local_attention(
+            qa, cache, cache, fb.block_tables, fb.seq_lens,
+            fb.query_start_locs, s.scale, 0, s.window, proj, -1, lat, 0, 1.0,
+            token_seq=fb.token_seq, tile_seq=fb.tile_seq, tile_q0=fb.tile_q0,
+            prefill_rows=fb.prefill_token_count)
+        sec = out[:, out_off:out_off + H * dv]
+        torch.bmm(lat.view(T, H, R).transpose(0, 1),
+                  self.uv.view(H, dv, R).transpose(1, 2),
+                  out=sec.view(T, H, dv).transpose(0, 1))
+        hops.sigmoid_gate_mul(sec, proj, off[tag + "g"])
+
+
+class MLSTM(nn.Module):
+    """mLSTM matrix memory with soft-capped exponential gating; q, k, v, the
+    output gate and both gate pre-activations are sections of the sublayer's
+    merged projection, the gate biases are added in fp32. The memory (with its
+    normaliser as an extra column) and the stabiliser live in the engine's
+    state cache."""
+
+    def __init__(self, spec: MLSTMMixerSpec, eps: float, layer_idx: int):
+        super().__init__()
+        self.spec = spec
+        self.eps = eps
+        self.layer_idx = layer_idx
+        f32 = torch.float32
+        self.i_bias = nn.Parameter(torch.zeros(spec.heads, dtype=f32))
+        self.f_bias = nn.Parameter(torch.zeros(spec.heads, dtype=f32))
+        self.norm_w = nn.Parameter(torch.ones(spec.heads * spec.vdim, dtype=f32))
+
+    def in_sections(self, tag: str):
+        s = self.spec
+        return [(tag + "q", s.heads * s.dim, False),
+                (tag + "k", s.heads * s.dim, False),
+                (tag + "v", s.heads * s.vdim, False),
+                (tag + "g", s.heads * s.vdim, False),
+                (tag + "i", s.heads, False),
+                (tag + "f", s.heads, False)]
+
+    @property
+    def out_width(self) -> int:
+        return self.spec.heads * self.spec.vdim
+
+    def kv_shape(self):
+        return None
+
+    def state_shape(self):
+        s = self.spec
+        return {"mem": (s.heads, s.dim, s.vdim + 1), "m": (s.heads,)}
+
+    def param_targets(self, prefix: str, ck: str):
+        s = self.spec
+        return {ck + ".i.b": (prefix + "i_bias", 0, 0, s.heads, 1.0),
+                ck + ".f.b": (prefix + "f_bias", 0, 0, s.heads, 1.0),
+                ck + ".norm": (prefix + "norm_w", 0, 0, s.heads * s.vdim, 1.0)}
+
+    def section_names(self, tag: str, ck: str):
+        return {tag + k: ck + "." + k for k in ("q", "k", "v", "g", "i", "f")}
+
+    def forward(self, proj: torch.Tensor, off: Dict[str, int], tag: str,
+                fb: ForwardBatch, kv: PagedKVCache, out: torch.Tensor,
+                out_off: int, out_scale: float) -> None:
+        s = self.spec
+        st = kv.state.named[self.layer_idx]
+        o, em = hops.mlstm_scan(
+            proj, off[tag + "q"], off[tag + "k"], off[tag + "v"],
+            off[tag + "i"], off[tag + "f"], s.heads, s.dim, s.vdim,
+            self.i_bias, self.f_bias, s.gate_cap, st["mem"], st["m"],
+            fb.state_slots, fb.query_start_locs, fb.seq_lens)
+        hops.mlstm_out(o, em, self.norm_w, proj, off[tag + "g"], self.eps,
+                       out, out_off)

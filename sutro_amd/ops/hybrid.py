@@ -102,11 +102,13 @@ def local_attention(q, k_cache, v_cache, block_tables, seq_lens,
                     query_start_locs, scale: float, chunk: int, window: int,
                     proj, gate_off: int, out, out_off: int, out_scale: float,
                     token_seq=None, tile_seq=None, tile_q0=None,
-                    prefill_rows: int = 0):
+                    prefill_rows: int = 0, bias_r1=None, bias_r2=None):
     """`tile_seq`/`tile_q0` (int32, 32 query rows a tile) cover the first
     `prefill_rows` rows: on the GPU in bf16 those rows run on the MFMA kernel
     when page size and head sizes allow it; the remaining (single-token) rows
-    and all other cases run on the generic one-wave-per-row kernel."""
+    and all other cases run on the generic one-wave-per-row kernel.
+    `bias_r1` / `bias_r2` (fp32 [H]): r1[h] * ln(1 + r2[h] * (i - j)) is taken
+    off the score of query i and key j."""
     if q.is_cuda:
         if tile_seq is None or tile_seq.numel() == 0:
             tile_seq = tile_q0 = None
@@ -115,11 +117,12 @@ def local_attention(q, k_cache, v_cache, block_tables, seq_lens,
                                block_tables, seq_lens, query_start_locs,
                                token_seq, scale, chunk, window, proj,
                                gate_off, out_scale, tile_seq, tile_q0,
-                               prefill_rows)
+                               prefill_rows, bias_r1, bias_r2)
         return
     torch_ref.local_attention(q, k_cache, v_cache, block_tables, seq_lens,
                               query_start_locs, scale, chunk, window, proj,
-                              gate_off, out, out_off, out_scale)
+                              gate_off, out, out_off, out_scale,
+                              bias_r1=bias_r1, bias_r2=bias_r2)
 
 
 def delta_prep(proj, q_off, k_off, v_off, b_off, a1_off, H, G, dk, dv,
@@ -173,3 +176,110 @@ def delta_out(o, norm_w, proj, g1_off: int, g2, eps: float, out,
         return
     torch_ref.delta_out(o, norm_w, proj, g1_off, g2, eps, out, out_off,
                         out_scale)
+
+
+# ---- hashed-bigram / sinusoid embedding, sandwich norms with depth-weighted
+# ---- sums, PolyNorm, tied-value attention prep, latent helpers, mLSTM ----
+
+sinusoid_inv_freq = torch_ref.sinusoid_inv_freq
+
+
+def token_embed(ids, prev_ids, positions, embed_w, bigram_w, buckets: int,
+                mul_prev: int, mul_cur: int, inv_freq, out=None):
+    """fp32 [T, W] sum of the token row, the hashed bigram row (row `buckets`
+    where prev_ids < 0) and the sinusoid of the position."""
+    if out is None:
+        out = torch.empty((ids.shape[0], embed_w.shape[1]),
+                          dtype=torch.float32, device=ids.device)
+    if ids.is_cuda:
+        _mix().token_embed(out, ids, prev_ids, positions, embed_w, bigram_w,
+                           buckets, mul_prev, mul_cur, inv_freq)
+    else:
+        out.copy_(torch_ref.token_embed(ids, prev_ids, positions, embed_w,
+                                        bigram_w, buckets, mul_prev, mul_cur,
+                                        inv_freq))
+    return out
+
+
+def weighted_rmsnorm(x, w, eps: float, out_dtype: torch.dtype):
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        _mix().weighted_rmsnorm(out, x, w, eps)
+        return out
+    return torch_ref.weighted_rmsnorm(x, w, eps, out_dtype)
+
+
+def norm_residual(x_in, y, w_post, eps: float, x_out, stack=None,
+                  depth_w=None, mix_out=None, next_w=None, h_out=None) -> None:
+    """x_out = x_in + n(y) * w_post; optionally the depth-weighted sum of the
+    first len(depth_w) entries of `stack` (the last of which is x_out) into
+    mix_out, and the next sublayer's normed input into h_out. One kernel."""
+    if x_in.is_cuda:
+        _mix().norm_residual(x_in, y, w_post, eps, x_out, stack, depth_w,
+                             mix_out, next_w, h_out)
+        return
+    torch_ref.norm_residual(x_in, y, w_post, eps, x_out, stack, depth_w,
+                            mix_out, next_w, h_out)
+
+
+def poly_act(z, coef, eps: float):
+    if z.is_cuda:
+        out = torch.empty_like(z)
+        _mix().poly_act(out, z, coef, eps)
+        return out
+    return torch_ref.poly_act(z, coef, eps)
+
+
+def tied_attn_prep(proj, q_off, k_off, H, G, dk, q_w, k_w, eps, positions,
+                   temp_coef: float, temp_every: int, slot_mapping, k_cache,
+                   v_cache):
+    if proj.is_cuda:
+        q = torch.empty((proj.shape[0], H, dk), dtype=proj.dtype,
+                        device=proj.device)
+        _mix().tied_attn_prep(q, proj, q_off, k_off, q_w, k_w, eps, positions,
+                              temp_coef, temp_every, slot_mapping, k_cache,
+                              v_cache)
+        return q
+    return torch_ref.tied_attn_prep(proj, q_off, k_off, H, G, dk, q_w, k_w,
+                                    eps, positions, temp_coef, temp_every,
+                                    slot_mapping, k_cache, v_cache)
+
+
+def section_rmsnorm(proj, off: int, n: int, w, eps: float, out,
+                    rows=None) -> None:
+    if proj.is_cuda:
+        _mix().section_rmsnorm(out, proj, off, w, eps, rows)
+        return
+    torch_ref.section_rmsnorm(proj, off, n, w, eps, out, rows)
+
+
+def sigmoid_gate_mul(v, proj, g_off: int) -> None:
+    if v.is_cuda:
+        _mix().sigmoid_gate_mul(v, proj, g_off)
+        return
+    torch_ref.sigmoid_gate_mul(v, proj, g_off)
+
+
+def mlstm_scan(proj, q_off, k_off, v_off, i_off, f_off, H, dk, dv, i_bias,
+               f_bias, cap: float, mem, mstate, state_slots, query_start_locs,
+               seq_lens):
+    if proj.is_cuda:
+        T = proj.shape[0]
+        o = torch.empty((T, H, dv + 1), dtype=torch.float32,
+                        device=proj.device)
+        em = torch.empty((T, H), dtype=torch.float32, device=proj.device)
+        _mix().mlstm_scan(o, em, proj, q_off, k_off, v_off, i_off, f_off,
+                          i_bias, f_bias, cap, mem, mstate, state_slots,
+                          query_start_locs, seq_lens)
+        return o, em
+    return torch_ref.mlstm_scan(proj, q_off, k_off, v_off, i_off, f_off, H,
+                                dk, dv, i_bias, f_bias, cap, mem, mstate,
+                                state_slots, query_start_locs, seq_lens)
+
+
+def mlstm_out(o, em, norm_w, proj, g_off: int, eps: float, out,
+              out_off: int) -> None:
+    if o.is_cuda:
+        _mix().mlstm_out(out, out_off, o, em, norm_w, proj, g_off, eps)
+        return
+    torch_ref.mlstm_out(o, em, norm_w, proj, g_off, eps, out, out_off)

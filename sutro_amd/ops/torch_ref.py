@@ -250,12 +250,14 @@ def attn_prep(proj, q_off, k_off, v_off, H, G, dk, dv, q_norm_w, k_norm_w,
 
 def local_attention(q, k_cache, v_cache, block_tables, seq_lens,
                     query_start_locs, scale, chunk, window, proj, gate_off,
-                    out, out_off, out_scale):
+                    out, out_off, out_scale, bias_r1=None, bias_r2=None):
     """Softmax attention of each sequence's new tokens over its cached keys
     under a local mask: query at position i sees j <= i with
     j >= (i // chunk) * chunk (chunk > 0) and j > i - window (window > 0).
     Head h's result is multiplied by out_scale * sigmoid(proj[t, gate_off+h])
-    (gate_off < 0: no gate) and written to out[t, out_off + h*dv : ...]."""
+    (gate_off < 0: no gate) and written to out[t, out_off + h*dv : ...].
+    With bias_r1 / bias_r2 (fp32 [H]) the score of query i and key j is
+    lowered by r1[h] * ln(1 + r2[h] * (i - j))."""
     T, H, dk = q.shape
     G, bs, dv = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
     rep = H // G
@@ -277,6 +279,10 @@ def local_attention(q, k_cache, v_cache, block_tables, seq_lens,
         kpos = torch.arange(L, device=q.device).unsqueeze(0)
         qpos = torch.arange(L - nq, L, device=q.device).unsqueeze(1)
         hidden = kpos > qpos
+        if bias_r1 is not None:
+            d = (qpos - kpos).clamp(min=0).to(torch.float32).unsqueeze(0)
+            scores = scores - bias_r1.float().view(H, 1, 1) * torch.log(
+                1.0 + bias_r2.float().view(H, 1, 1) * d)
         if chunk > 0:
             hidden = hidden | (kpos < (qpos // chunk) * chunk)
         if window > 0:
@@ -383,3 +389,173 @@ def delta_out(o, norm_w, proj, g1_off, g2, eps, out, out_off, out_scale):
     gate = torch.sigmoid(proj[:, g1_off:g1_off + r].float() @ g2.float().T).view(T, H, dv)
     y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()
     out[:, out_off:out_off + H * dv] = (y * gate * out_scale).reshape(T, H * dv).to(out.dtype)
+
+
+# --------------------------------------------------------------------------
+# More mechanisms of layer-list decoders: hashed-bigram + sinusoid embedding,
+# weighted RMS norms around a sublayer with a depth-weighted sum of all earlier
+# layer results, PolyNorm, windowed attention with whole-projection q/k norm /
+# position-dependent query temperature / logarithmic distance bias, latent
+# attention helpers, and the mLSTM matrix memory.
+# --------------------------------------------------------------------------
+
+
+def sinusoid_inv_freq(width: int, base: float) -> torch.Tensor:
+    """fp32 [width/2]: base^(-2i/width), rounded once from fp64."""
+    i = torch.arange(width // 2, dtype=torch.float64)
+    return (float(base) ** (-2.0 * i / width)).float()
+
+
+def token_embed(ids, prev_ids, positions, embed_w, bigram_w, buckets: int,
+                mul_prev: int, mul_cur: int, inv_freq):
+    """fp32 [T, W]: embed[id] (+ bigram[(prev*mul_prev + id*mul_cur) mod
+    buckets], row `buckets` where prev < 0) (+ the sinusoid of the position:
+    column 2i = sin(p * inv_freq[i]), column 2i+1 = cos of the same fp32
+    angle)."""
+    x = embed_w[ids].float()
+    if bigram_w is not None:
+        row = (prev_ids * mul_prev + ids * mul_cur) % buckets
+        row = torch.where(prev_ids < 0, torch.full_like(row, buckets), row)
+        x = x + bigram_w[row].float()
+    if inv_freq is not None:
+        ang = positions.to(torch.float32).unsqueeze(1) * inv_freq.unsqueeze(0)
+        x = x + torch.stack([ang.sin(), ang.cos()], dim=-1).reshape(x.shape[0], -1)
+    return x
+
+
+def _unit_rms(x: torch.Tensor, eps: float) -> torch.Tensor:
+    return x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+
+
+def weighted_rmsnorm(x, w, eps: float, out_dtype: torch.dtype):
+    return (_unit_rms(x.float(), eps) * w.float()).to(out_dtype)
+
+
+def norm_residual(x_in, y, w_post, eps: float, x_out, stack=None,
+                  depth_w=None, mix_out=None, next_w=None, h_out=None) -> None:
+    """r = x_in + n(y) * w_post -> x_out (fp32; may be x_in itself). With
+    `depth_w` [n]: z = sum_j depth_w[j] * stack[j] over the first n entries of
+    `stack` [*, T, W], whose entry n-1 is x_out, -> mix_out; else z = r. With
+    `next_w`: h_out = n(z) * next_w in h_out's dtype. n divides a row by its
+    root mean square (eps inside the root)."""
+    r = x_in + _unit_rms(y.float(), eps) * w_post.float()
+    x_out.copy_(r)
+    z = r
+    if depth_w is not None:
+        n = depth_w.numel()
+        z = (depth_w.float().view(n, 1, 1) * stack[:n]).sum(0)
+        mix_out.copy_(z)
+    if next_w is not None:
+        h_out.copy_((_unit_rms(z, eps) * next_w.float()).to(h_out.dtype))
+
+
+def poly_act(z, coef, eps: float):
+    """coef[0] n(z) + coef[1] n(z^2) + coef[2] n(z^3) + coef[3], powers taken
+    element by element, n as above over the row."""
+    zf = z.float()
+    c = coef.float()
+    z2 = zf * zf
+    z3 = z2 * zf
+    y = (c[0] * _unit_rms(zf, eps) + c[1] * _unit_rms(z2, eps)
+         + c[2] * _unit_rms(z3, eps) + c[3])
+    return y.to(z.dtype)
+
+
+def tied_attn_prep(proj, q_off, k_off, H, G, dk, q_w, k_w, eps, positions,
+                   temp_coef: float, temp_every: int, slot_mapping, k_cache,
+                   v_cache):
+    """Queries and keys of attention whose values are its raw keys: the q and
+    k sections of `proj` are each RMS-normed over the WHOLE section (all heads
+    at once) with weights q_w / k_w; q is then scaled by 1 + temp_coef *
+    ln(floor((p + 1) / temp_every) + 1) at position p (temp_every <= 0: no
+    scaling). The normed k goes to k_cache, the raw k section to v_cache.
+    Returns q [T, H, dk]."""
+    T = proj.shape[0]
+    q = proj[:, q_off:q_off + H * dk].float()
+    k = proj[:, k_off:k_off + G * dk]
+    q = _unit_rms(q, eps) * q_w.float()
+    kn = _unit_rms(k.float(), eps) * k_w.float()
+    if temp_every > 0:
+        p = positions.to(torch.float32)
+        q = q * (1.0 + temp_coef * torch.log(
+            torch.floor((p + 1.0) / float(temp_every)) + 1.0)).unsqueeze(1)
+    bs = k_cache.shape[2]
+    blk = slot_mapping // bs
+    off = slot_mapping % bs
+    k_cache[blk, :, off] = kn.reshape(T, G, dk).to(k_cache.dtype)
+    v_cache[blk, :, off] = k.reshape(T, G, dk).to(v_cache.dtype)
+    return q.reshape(T, H, dk).to(proj.dtype)
+
+
+def section_rmsnorm(proj, off: int, n: int, w, eps: float, out, rows=None):
+    """out[rows[t] or t] = n(proj[t, off:off+n]) * w; `out` is [N, n]."""
+    y = (_unit_rms(proj[:, off:off + n].float(), eps) * w.float()).to(out.dtype)
+    if rows is None:
+        out.copy_(y)
+    else:
+        out[rows] = y
+
+
+def sigmoid_gate_mul(v, proj, g_off: int) -> None:
+    """v [T, N] *= sigmoid(proj[:, g_off:g_off+N]), in place."""
+    N = v.shape[1]
+    v.copy_((v.float() * torch.sigmoid(proj[:, g_off:g_off + N].float())).to(v.dtype))
+
+
+def mlstm_scan(proj, q_off, k_off, v_off, i_off, f_off, H, dk, dv, i_bias,
+               f_bias, cap: float, mem, mstate, state_slots, query_start_locs,
+               seq_lens):
+    """mLSTM matrix memory over every sequence's new tokens.
+
+    Per head, with log gates i = cap*tanh((a_i + b_i)/cap) and f =
+    logsigmoid(cap*tanh((a_f + b_f)/cap)) (a_* = the i/f sections of `proj`)
+    and the running maximum m (0 at a sequence's start):
+        m' = max(f + m, i);  C <- exp(f + m - m') C + exp(i - m') k [v, 1]^T
+    where C [dk, dv+1] carries the normaliser n as its last column
+    (mem[slot, h]), m lives in mstate[slot, h], q is scaled by dk^-1/2.
+    Returns (C^T q [T, H, dv+1] fp32, exp(-m') [T, H] fp32)."""
+    T = proj.shape[0]
+    q = proj[:, q_off:q_off + H * dk].float().reshape(T, H, dk) * (float(dk) ** -0.5)
+    k = proj[:, k_off:k_off + H * dk].float().reshape(T, H, dk)
+    v = proj[:, v_off:v_off + H * dv].float().reshape(T, H, dv)
+    v1 = torch.cat([v, torch.ones(T, H, 1, dtype=torch.float32, device=v.device)], -1)
+    ig = cap * torch.tanh((proj[:, i_off:i_off + H].float() + i_bias.float()) / cap)
+    fg = torch.nn.functional.logsigmoid(
+        cap * torch.tanh((proj[:, f_off:f_off + H].float() + f_bias.float()) / cap))
+    o = torch.empty(T, H, dv + 1, dtype=torch.float32, device=proj.device)
+    em = torch.empty(T, H, dtype=torch.float32, device=proj.device)
+    for s in range(seq_lens.numel()):
+        a, b = int(query_start_locs[s]), int(query_start_locs[s + 1])
+        n = b - a
+        if n == 0:
+            continue
+        start = int(seq_lens[s]) - n
+        slot = int(state_slots[s])
+        if start > 0:
+            C, m = mem[slot].clone(), mstate[slot].clone()
+        else:
+            C, m = torch.zeros_like(mem[slot]), torch.zeros_like(mstate[slot])
+        for t in range(a, b):
+            mn = torch.maximum(fg[t] + m, ig[t])
+            fa = torch.exp(fg[t] + m - mn)
+            ib = torch.exp(ig[t] - mn)
+            C = fa.view(H, 1, 1) * C + (ib.view(H, 1) * k[t]).unsqueeze(-1) * v1[t].unsqueeze(1)
+            m = mn
+            o[t] = torch.einsum("hkv,hk->hv", C, q[t])
+            em[t] = torch.exp(-m)
+        mem[slot] = C
+        mstate[slot] = m
+    return o, em
+
+
+def mlstm_out(o, em, norm_w, proj, g_off: int, eps: float, out, out_off: int):
+    """h = o[..., :dv] / (max(|o[..., dv]|, em) + 1e-6); each head of h divided
+    by its root mean square; times norm_w [H*dv] and sigmoid of the gate
+    section of `proj`; written to out[:, out_off : out_off + H*dv]."""
+    T, H, dv1 = o.shape
+    dv = dv1 - 1
+    den = torch.maximum(o[..., dv].abs(), em) + 1e-6
+    h = o[..., :dv] / den.unsqueeze(-1)
+    h = _unit_rms(h, eps).reshape(T, H * dv) * norm_w.float()
+    h = h * torch.sigmoid(proj[:, g_off:g_off + H * dv].float())
+    out[:, out_off:out_off + H * dv] = h.to(out.dtype)

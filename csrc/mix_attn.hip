@@ -6,7 +6,9 @@
 //                    made once per step), K/V scatter into the paged caches,
 //                    q out.
 //   local_attention  softmax attention of every new token over the cached
-//                    keys its mask lets it see, times a per-head sigmoid gate.
+//                    keys its mask lets it see, times a per-head sigmoid gate;
+//                    optionally r1[h] * ln(1 + r2[h] * distance) is taken off
+//                    every score (per-head logarithmic distance bias).
 //
 // Cache layout per layer: K [blocks, G, page, dk], V [blocks, G, page, dv].
 // Mask of a query at position p: keys j in [lo, p],
@@ -211,7 +213,8 @@ __global__ void local_attention_kernel(
     const int* __restrict__ bt, int bt_stride, const int* __restrict__ seq_lens,
     const int* __restrict__ qlocs, const int* __restrict__ token_seq,
     float scale, int chunk, int window, const A* __restrict__ proj, long ld,
-    int gate_off, float out_scale, long t0, long T, int H, int G, int dk,
+    int gate_off, float out_scale, const float* __restrict__ bias_r1,
+    const float* __restrict__ bias_r2, long t0, long T, int H, int G, int dk,
     int dv, int page) {
   extern __shared__ float sm[];  // WPB * dk floats: the wave's query
   const int lane = threadIdx.x & (WAVE - 1);
@@ -233,6 +236,9 @@ __global__ void local_attention_kernel(
   if (chunk > 0) lo = (p / chunk) * chunk;
   if (window > 0 && p - window + 1 > lo) lo = p - window + 1;
   const int* table = bt + (long)s * bt_stride;
+  // distance bias: r1 * ln(1 + r2 * (p - j)) is taken off the score
+  const float r1 = bias_r1 ? bias_r1[h] : 0.f;
+  const float r2 = bias_r1 ? bias_r2[h] : 0.f;
 
   float m = -INFINITY, l = 0.f;
   float acc[NV];
@@ -251,6 +257,7 @@ __global__ void local_attention_kernel(
       float dot = 0.f;
       for (int i = 0; i < dk; ++i) dot += qs[i] * ldf<A>(kr + i);
       sc = dot * scale;
+      if (bias_r1) sc -= r1 * logf(1.f + r2 * (float)(p - j));
     }
     const float m_new = fmaxf(m, wave_max_f32(sc));
     const float pj = live ? expf(sc - m_new) : 0.f;
@@ -332,7 +339,8 @@ static void launch_local_attention(
     const void* v_cache, const int* bt, int bt_stride, const int* seq_lens,
     const int* qlocs, const int* token_seq, float scale, int chunk,
     int window, const void* proj, long ld, int gate_off, float out_scale,
-    long t0, long T, int H, int G, int dk, int dv, int page, hipStream_t s) {
+    const float* bias_r1, const float* bias_r2, long t0, long T, int H, int G,
+    int dk, int dv, int page, hipStream_t s) {
   const long units = T * H;
   const int grid = (int)((units + WPB - 1) / WPB);
   if (grid == 0) return;
@@ -342,11 +350,12 @@ static void launch_local_attention(
                      dim3(WPB * WAVE), smem, s, (A*)out, ldo, out_off,       \
                      (const A*)q, (const A*)k_cache, (const A*)v_cache, bt,  \
                      bt_stride, seq_lens, qlocs, token_seq, scale, chunk,    \
-                     window, (const A*)proj, ld, gate_off, out_scale, t0, T, \
-                     H, G, dk, dv, page)
+                     window, (const A*)proj, ld, gate_off, out_scale,        \
+                     bias_r1, bias_r2, t0, T, H, G, dk, dv, page)
   if (dv <= 64) LAUNCH_LA(1);
   else if (dv <= 128) LAUNCH_LA(2);
-  else LAUNCH_LA(4);
+  else if (dv <= 256) LAUNCH_LA(4);
+  else LAUNCH_LA(8);
 #undef LAUNCH_LA
 }
 
@@ -355,16 +364,18 @@ extern "C" void mix_local_attention(
     const void* v_cache, const int* bt, int bt_stride, const int* seq_lens,
     const int* qlocs, const int* token_seq, float scale, int chunk,
     int window, const void* proj, long ld, int gate_off, float out_scale,
-    long t0, long T, int H, int G, int dk, int dv, int page, int f32,
-    hipStream_t s) {
+    const float* bias_r1, const float* bias_r2, long t0, long T, int H, int G,
+    int dk, int dv, int page, int f32, hipStream_t s) {
   if (f32)
     launch_local_attention<float>(out, ldo, out_off, q, k_cache, v_cache, bt,
                                   bt_stride, seq_lens, qlocs, token_seq, scale,
                                   chunk, window, proj, ld, gate_off, out_scale,
-                                  t0, T, H, G, dk, dv, page, s);
+                                  bias_r1, bias_r2, t0, T, H, G, dk, dv, page,
+                                  s);
   else
     launch_local_attention<u16>(out, ldo, out_off, q, k_cache, v_cache, bt,
                                 bt_stride, seq_lens, qlocs, token_seq, scale,
                                 chunk, window, proj, ld, gate_off, out_scale,
-                                t0, T, H, G, dk, dv, page, s);
+                                bias_r1, bias_r2, t0, T, H, G, dk, dv, page,
+                                s);
 }

@@ -9,6 +9,8 @@
 //   - a per-row lower key bound lo(p) = max(chunk ? p/chunk*chunk : 0,
 //     window ? p - window + 1 : 0): pages wholly below the bound of the
 //     tile's first row are never read; masked scores contribute exactly 0,
+//   - an optional per-head distance bias r1 * ln(1 + r2 * (p - j)) taken off
+//     the scaled score,
 //   - score scale from the caller, per-head sigmoid output gate and output
 //     scale in the epilogue, output written into a column section of the
 //     merged output-projection input.
@@ -45,7 +47,8 @@ __global__ void local_attention_mfma_kernel(
     const int* __restrict__ bt, int bt_stride, const int* __restrict__ seq_lens,
     const int* __restrict__ qlocs, const int* __restrict__ tile_seq,
     const int* __restrict__ tile_q0, float scale, int chunk, int window,
-    const u16* __restrict__ proj, long ld, int gate_off, float out_scale, int H,
+    const u16* __restrict__ proj, long ld, int gate_off, float out_scale,
+    const float* __restrict__ bias_r1, const float* __restrict__ bias_r2, int H,
     int Hk, int dk, int dv) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int w = threadIdx.x / WAVE;
@@ -93,6 +96,9 @@ __global__ void local_attention_mfma_kernel(
 #pragma unroll
   for (int b = 0; b < DVP / 32; ++b) acc[b] = (f32x16)(0.f);
   float m_run = -1e30f, l_run = 0.f;
+  // distance bias of this wave's head: r1 * ln(1 + r2 * (p - j))
+  const float r1 = bias_r1 ? bias_r1[hq] : 0.f;
+  const float r2 = bias_r1 ? bias_r2[hq] : 0.f;
 
   const int kt0 = lo_tile / PG, kt1 = (kv_end + PG - 1) / PG;
   for (int kt = kt0; kt < kt1; ++kt) {
@@ -134,7 +140,9 @@ __global__ void local_attention_mfma_kernel(
     for (int r = 0; r < 16; ++r) {
       const int kvpos = kv0 + drow(r, hi);
       vis[r] = kvpos <= my_p && kvpos >= lo_row;
-      sc[r] = vis[r] ? d1[r] * scale : -1e30f;
+      float sv = d1[r] * scale;
+      if (bias_r1) sv -= r1 * logf(1.f + r2 * (float)max(my_p - kvpos, 0));
+      sc[r] = vis[r] ? sv : -1e30f;
       tmax = fmaxf(tmax, sc[r]);
     }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
@@ -211,8 +219,8 @@ extern "C" int mix_local_attention_mfma(
     const void* v_cache, const int* bt, int bt_stride, const int* seq_lens,
     const int* qlocs, const int* tile_seq, const int* tile_q0, int n_tiles,
     float scale, int chunk, int window, const void* proj, long ld,
-    int gate_off, float out_scale, int H, int Hk, int dk, int dv, int page,
-    hipStream_t s) {
+    int gate_off, float out_scale, const float* bias_r1, const float* bias_r2,
+    int H, int Hk, int dk, int dv, int page, hipStream_t s) {
   if (page != PG || dk % 8 || dv % 8 || dk > 256 || dv > 256 || H % Hk)
     return 0;
   const int G = H / Hk;
@@ -229,7 +237,8 @@ extern "C" int mix_local_attention_mfma(
                      ldo, out_off, (const u16*)q, (const u16*)k_cache,        \
                      (const u16*)v_cache, bt, bt_stride, seq_lens, qlocs,     \
                      tile_seq, tile_q0, scale, chunk, window,                 \
-                     (const u16*)proj, ld, gate_off, out_scale, H, Hk, dk, dv)
+                     (const u16*)proj, ld, gate_off, out_scale, bias_r1,     \
+                     bias_r2, H, Hk, dk, dv)
   if (DKP == 64) {
     if (DVP == 64) LAUNCH_M(64, 64);
     else if (DVP == 128) LAUNCH_M(64, 128);

@@ -49,13 +49,39 @@ void mix_attn_prep(void*, const void*, long, int, int, int, const float*,
 void mix_local_attention(void*, long, int, const void*, const void*,
                          const void*, const int*, int, const int*, const int*,
                          const int*, float, int, int, const void*, long, int,
-                         float, long, long, int, int, int, int, int, int,
-                         hipStream_t);
+                         float, const float*, const float*, long, long, int,
+                         int, int, int, int, int, hipStream_t);
 int mix_local_attention_mfma(void*, long, int, const void*, const void*,
                              const void*, const int*, int, const int*,
                              const int*, const int*, const int*, int, float,
-                             int, int, const void*, long, int, float, int, int,
-                             int, int, int, hipStream_t);
+                             int, int, const void*, long, int, float,
+                             const float*, const float*, int, int, int, int,
+                             int, hipStream_t);
+void mix_token_embed(float*, const long*, const long*, const long*,
+                     const void*, const void*, long, long, long, const float*,
+                     long, int, int, hipStream_t);
+void mix_weighted_rmsnorm(void*, const float*, const float*, float, long, int,
+                          int, hipStream_t);
+void mix_norm_residual(const float*, const void*, const float*, float, float*,
+                       const float*, long, const float*, int, float*,
+                       const float*, void*, long, int, int, hipStream_t);
+void mix_poly_act(void*, const void*, const float*, float, long, int, int,
+                  hipStream_t);
+void mix_tied_attn_prep(void*, const void*, long, int, int, const float*,
+                        const float*, float, const long*, float, int,
+                        const long*, void*, void*, long, int, int, int, int,
+                        int, hipStream_t);
+void mix_section_rmsnorm(void*, long, const void*, long, int, const float*,
+                         float, const long*, long, int, int, hipStream_t);
+void mix_sigmoid_gate_mul(void*, long, const void*, long, int, long, int, int,
+                          hipStream_t);
+void mix_mlstm_scan(float*, float*, float*, float*, const void*, long, int,
+                    int, int, int, int, const float*, const float*, float,
+                    float*, float*, const int*, const int*, const int*, int,
+                    int, int, int, int, hipStream_t);
+void mix_mlstm_out(void*, long, int, const float*, const float*, const float*,
+                   const void*, long, int, float, long, int, int, int,
+                   hipStream_t);
 void mix_delta_prep(float*, float*, float*, float*, float*, const void*, long,
                     int, int, int, int, int, const float*, const float*, int,
                     const float*,
@@ -168,7 +194,8 @@ void local_attention(torch::Tensor out, long out_off, torch::Tensor q,
                      long gate_off, double out_scale,
                      c10::optional<torch::Tensor> tile_seq,
                      c10::optional<torch::Tensor> tile_q0,
-                     long prefill_rows) {
+                     long prefill_rows, c10::optional<torch::Tensor> bias_r1,
+                     c10::optional<torch::Tensor> bias_r2) {
   CHECK_GPU(q); CHECK_CONTIG(q); CHECK_CONTIG(k_cache); CHECK_CONTIG(v_cache);
   CHECK_I32(bt); CHECK_I32(seq_lens); CHECK_I32(qlocs); CHECK_I32(token_seq);
   CHECK_CONTIG(bt);
@@ -177,7 +204,16 @@ void local_attention(torch::Tensor out, long out_off, torch::Tensor q,
   const long dv = v_cache.size(3);
   TORCH_CHECK(k_cache.size(3) == dk, "key size mismatch");
   TORCH_CHECK(H % G == 0, "heads must be a multiple of kv heads");
-  TORCH_CHECK(dv <= 256 && dk <= 4096, "unsupported head sizes");
+  TORCH_CHECK(dv <= 512 && dk <= 4096, "unsupported head sizes");
+  const float* r1 = nullptr; const float* r2 = nullptr;
+  if (bias_r1.has_value()) {
+    TORCH_CHECK(bias_r2.has_value(), "distance bias needs r1 and r2");
+    CHECK_GPU(*bias_r1); CHECK_F32(*bias_r1); CHECK_CONTIG(*bias_r1);
+    CHECK_GPU(*bias_r2); CHECK_F32(*bias_r2); CHECK_CONTIG(*bias_r2);
+    TORCH_CHECK(bias_r1->numel() == H && bias_r2->numel() == H,
+                "distance bias: one r1 and r2 per head");
+    r1 = bias_r1->data_ptr<float>(); r2 = bias_r2->data_ptr<float>();
+  }
   TORCH_CHECK(out.dim() == 2 && out.stride(1) == 1 && out.size(0) == T &&
               out_off >= 0 && out_off + H * dv <= out.size(1), "out section");
   TORCH_CHECK(out.scalar_type() == q.scalar_type() &&
@@ -204,7 +240,7 @@ void local_attention(torch::Tensor out, long out_off, torch::Tensor q,
             tile_seq->data_ptr<int>(), tile_q0->data_ptr<int>(),
             (int)tile_seq->numel(), (float)scale, (int)chunk, (int)window,
             proj.data_ptr(), proj.stride(0), (int)gate_off, (float)out_scale,
-            (int)H, (int)G, (int)dk, (int)dv, (int)page, cur_stream()))
+            r1, r2, (int)H, (int)G, (int)dk, (int)dv, (int)page, cur_stream()))
       t0 = prefill_rows;
   }
   if (t0 < T)
@@ -214,7 +250,8 @@ void local_attention(torch::Tensor out, long out_off, torch::Tensor q,
                         seq_lens.data_ptr<int>(), qlocs.data_ptr<int>(),
                         token_seq.data_ptr<int>(), (float)scale, (int)chunk,
                         (int)window, proj.data_ptr(), proj.stride(0),
-                        (int)gate_off, (float)out_scale, t0, T - t0, (int)H,
+                        (int)gate_off, (float)out_scale, r1, r2, t0, T - t0,
+                        (int)H,
                         (int)G, (int)dk, (int)dv, (int)page, act_kind(q),
                         cur_stream());
 }
@@ -326,6 +363,242 @@ void delta_out(torch::Tensor out, long out_off, torch::Tensor o,
                 act_kind(out), cur_stream());
 }
 
+// ---- embedding, sandwich norms with depth-weighted sums, PolyNorm ----
+
+void token_embed(torch::Tensor out, torch::Tensor ids,
+                 c10::optional<torch::Tensor> prev, torch::Tensor pos,
+                 torch::Tensor embed, c10::optional<torch::Tensor> bigram,
+                 long buckets, long mul_prev, long mul_cur,
+                 c10::optional<torch::Tensor> inv_freq) {
+  CHECK_GPU(out); CHECK_F32(out); CHECK_CONTIG(out); CHECK_GPU(ids);
+  CHECK_I64(ids); CHECK_I64(pos); CHECK_CONTIG(ids); CHECK_CONTIG(pos);
+  CHECK_GPU(embed); CHECK_CONTIG(embed);
+  const long T = ids.numel(), W = embed.size(1);
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == W &&
+              pos.numel() == T, "embedding output shape");
+  const void* bp = nullptr; const long* pp = nullptr;
+  if (bigram.has_value()) {
+    TORCH_CHECK(prev.has_value(), "a bigram table needs the previous tokens");
+    CHECK_GPU(*bigram); CHECK_CONTIG(*bigram); CHECK_I64(*prev);
+    CHECK_CONTIG(*prev);
+    TORCH_CHECK(bigram->scalar_type() == embed.scalar_type() &&
+                bigram->size(1) == W && bigram->size(0) == buckets + 1 &&
+                prev->numel() == T && buckets > 0, "bigram table shape");
+    bp = bigram->data_ptr(); pp = prev->data_ptr<long>();
+  }
+  const float* fp = nullptr;
+  if (inv_freq.has_value()) {
+    CHECK_GPU(*inv_freq); CHECK_F32(*inv_freq); CHECK_CONTIG(*inv_freq);
+    TORCH_CHECK(W % 2 == 0 && inv_freq->numel() == W / 2, "sinusoid table");
+    fp = inv_freq->data_ptr<float>();
+  }
+  mix_token_embed(out.data_ptr<float>(), ids.data_ptr<long>(), pp,
+                  pos.data_ptr<long>(), embed.data_ptr(), bp, buckets,
+                  mul_prev, mul_cur, fp, T, (int)W, act_kind(embed),
+                  cur_stream());
+}
+
+void weighted_rmsnorm(torch::Tensor out, torch::Tensor x, torch::Tensor w,
+                      double eps) {
+  CHECK_GPU(x); CHECK_CONTIG(x); CHECK_F32(x); CHECK_GPU(out);
+  CHECK_CONTIG(out); CHECK_GPU(w); CHECK_F32(w); CHECK_CONTIG(w);
+  const long W = x.size(-1), T = x.numel() / W;
+  TORCH_CHECK(out.numel() == x.numel() && w.numel() == W, "norm shapes");
+  mix_weighted_rmsnorm(out.data_ptr(), x.data_ptr<float>(),
+                       w.data_ptr<float>(), (float)eps, T, (int)W,
+                       act_kind(out), cur_stream());
+}
+
+void norm_residual(torch::Tensor x_in, torch::Tensor y, torch::Tensor w_post,
+                   double eps, torch::Tensor x_out,
+                   c10::optional<torch::Tensor> stack,
+                   c10::optional<torch::Tensor> depth_w,
+                   c10::optional<torch::Tensor> mix_out,
+                   c10::optional<torch::Tensor> next_w,
+                   c10::optional<torch::Tensor> h_out) {
+  CHECK_GPU(x_in); CHECK_F32(x_in); CHECK_CONTIG(x_in);
+  CHECK_GPU(x_out); CHECK_F32(x_out); CHECK_CONTIG(x_out);
+  CHECK_GPU(y); CHECK_CONTIG(y); CHECK_GPU(w_post); CHECK_F32(w_post);
+  CHECK_CONTIG(w_post);
+  TORCH_CHECK(x_in.dim() == 2, "x_in must be [T, W]");
+  const long T = x_in.size(0), W = x_in.size(1);
+  TORCH_CHECK(y.dim() == 2 && y.size(0) == T && y.size(1) == W &&
+              x_out.numel() == T * W && w_post.numel() == W, "row shapes");
+  const float* sp = nullptr; const float* dp = nullptr; float* mp = nullptr;
+  long stride = 0; int nd = 0;
+  if (depth_w.has_value()) {
+    TORCH_CHECK(stack.has_value() && mix_out.has_value(),
+                "a depth-weighted sum needs the kept results and an output");
+    CHECK_GPU(*stack); CHECK_F32(*stack); CHECK_CONTIG(*stack);
+    CHECK_GPU(*depth_w); CHECK_F32(*depth_w); CHECK_CONTIG(*depth_w);
+    CHECK_GPU(*mix_out); CHECK_F32(*mix_out); CHECK_CONTIG(*mix_out);
+    nd = (int)depth_w->numel();
+    TORCH_CHECK(stack->dim() == 3 && stack->size(1) == T &&
+                stack->size(2) == W && nd >= 1 && stack->size(0) >= nd &&
+                mix_out->numel() == T * W, "kept-results shape");
+    // the newest kept result is the row this call writes
+    TORCH_CHECK(x_out.data_ptr<float>() ==
+                stack->data_ptr<float>() + (long)(nd - 1) * T * W,
+                "x_out must be entry len(depth_w)-1 of the kept results");
+    sp = stack->data_ptr<float>(); dp = depth_w->data_ptr<float>();
+    mp = mix_out->data_ptr<float>(); stride = T * W;
+  }
+  const float* np_ = nullptr; void* hp = nullptr;
+  if (next_w.has_value()) {
+    TORCH_CHECK(h_out.has_value(), "next_w needs h_out");
+    CHECK_GPU(*next_w); CHECK_F32(*next_w); CHECK_CONTIG(*next_w);
+    CHECK_GPU(*h_out); CHECK_CONTIG(*h_out);
+    TORCH_CHECK(next_w->numel() == W && h_out->numel() == T * W &&
+                h_out->scalar_type() == y.scalar_type(), "h_out shape");
+    np_ = next_w->data_ptr<float>(); hp = h_out->data_ptr();
+  }
+  mix_norm_residual(x_in.data_ptr<float>(), y.data_ptr(),
+                    w_post.data_ptr<float>(), (float)eps,
+                    x_out.data_ptr<float>(), sp, stride, dp, nd, mp, np_, hp,
+                    T, (int)W, act_kind(y), cur_stream());
+}
+
+void poly_act(torch::Tensor out, torch::Tensor z, torch::Tensor coef,
+              double eps) {
+  CHECK_GPU(z); CHECK_CONTIG(z); CHECK_GPU(out); CHECK_CONTIG(out);
+  CHECK_GPU(coef); CHECK_F32(coef); CHECK_CONTIG(coef);
+  TORCH_CHECK(z.dim() == 2 && out.sizes() == z.sizes() &&
+              out.scalar_type() == z.scalar_type() && coef.numel() == 4,
+              "activation shapes");
+  mix_poly_act(out.data_ptr(), z.data_ptr(), coef.data_ptr<float>(),
+               (float)eps, z.size(0), (int)z.size(1), act_kind(z),
+               cur_stream());
+}
+
+// ---- whole-projection norms: tied-value attention prep, latents, gates ----
+
+void tied_attn_prep(torch::Tensor q_out, torch::Tensor proj, long q_off,
+                    long k_off, torch::Tensor q_w, torch::Tensor k_w,
+                    double eps, torch::Tensor pos, double temp_coef,
+                    long temp_every, torch::Tensor slots,
+                    torch::Tensor k_cache, torch::Tensor v_cache) {
+  CHECK_GPU(proj); CHECK_GPU(q_out); CHECK_CONTIG(q_out);
+  CHECK_GPU(k_cache); CHECK_GPU(v_cache);
+  CHECK_CONTIG(k_cache); CHECK_CONTIG(v_cache);
+  CHECK_I64(slots); CHECK_I64(pos); CHECK_CONTIG(slots); CHECK_CONTIG(pos);
+  CHECK_GPU(q_w); CHECK_F32(q_w); CHECK_CONTIG(q_w);
+  CHECK_GPU(k_w); CHECK_F32(k_w); CHECK_CONTIG(k_w);
+  const long T = q_out.size(0), H = q_out.size(1), dk = q_out.size(2);
+  const long G = k_cache.size(1), page = k_cache.size(2);
+  TORCH_CHECK(k_cache.dim() == 4 && k_cache.size(3) == dk &&
+              v_cache.sizes() == k_cache.sizes(),
+              "values are the keys: both caches must be [blocks, G, page, dk]");
+  TORCH_CHECK(q_out.scalar_type() == proj.scalar_type() &&
+              k_cache.scalar_type() == proj.scalar_type() &&
+              v_cache.scalar_type() == proj.scalar_type(),
+              "q, caches and projections must share one dtype");
+  TORCH_CHECK(proj.size(0) == T && slots.numel() == T && pos.numel() == T,
+              "row mismatch");
+  TORCH_CHECK(q_w.numel() == H * dk && k_w.numel() == G * dk, "norm sizes");
+  check_proj(proj, q_off, H * dk, "q");
+  check_proj(proj, k_off, G * dk, "k");
+  mix_tied_attn_prep(q_out.data_ptr(), proj.data_ptr(), proj.stride(0),
+                     (int)q_off, (int)k_off, q_w.data_ptr<float>(),
+                     k_w.data_ptr<float>(), (float)eps, pos.data_ptr<long>(),
+                     (float)temp_coef, (int)temp_every, slots.data_ptr<long>(),
+                     k_cache.data_ptr(), v_cache.data_ptr(), T, (int)H, (int)G,
+                     (int)dk, (int)page, act_kind(proj), cur_stream());
+}
+
+void section_rmsnorm(torch::Tensor out, torch::Tensor proj, long off,
+                     torch::Tensor w, double eps,
+                     c10::optional<torch::Tensor> rows) {
+  CHECK_GPU(proj); CHECK_GPU(out); CHECK_GPU(w); CHECK_F32(w); CHECK_CONTIG(w);
+  TORCH_CHECK(out.dim() == 2 && out.stride(1) == 1 &&
+              out.scalar_type() == proj.scalar_type(), "out must be [N, n] rows");
+  const long T = proj.size(0), n = out.size(1);
+  TORCH_CHECK(w.numel() == n, "norm size");
+  check_proj(proj, off, n, "normed");
+  const long* rp = nullptr;
+  if (rows.has_value()) {
+    CHECK_GPU(*rows); CHECK_I64(*rows); CHECK_CONTIG(*rows);
+    TORCH_CHECK(rows->numel() == T, "one destination row per token");
+    rp = rows->data_ptr<long>();
+  } else {
+    TORCH_CHECK(out.size(0) == T, "row mismatch");
+  }
+  mix_section_rmsnorm(out.data_ptr(), out.stride(0), proj.data_ptr(),
+                      proj.stride(0), (int)off, w.data_ptr<float>(),
+                      (float)eps, rp, T, (int)n, act_kind(proj), cur_stream());
+}
+
+void sigmoid_gate_mul(torch::Tensor v, torch::Tensor proj, long g_off) {
+  CHECK_GPU(v); CHECK_GPU(proj);
+  TORCH_CHECK(v.dim() == 2 && v.stride(1) == 1 &&
+              v.scalar_type() == proj.scalar_type() &&
+              proj.size(0) == v.size(0), "gated rows");
+  check_proj(proj, g_off, v.size(1), "gate");
+  mix_sigmoid_gate_mul(v.data_ptr(), v.stride(0), proj.data_ptr(),
+                       proj.stride(0), (int)g_off, v.size(0), (int)v.size(1),
+                       act_kind(v), cur_stream());
+}
+
+// ---- mLSTM ----
+
+void mlstm_scan(torch::Tensor o, torch::Tensor em, torch::Tensor proj,
+                long q_off, long k_off, long v_off, long i_off, long f_off,
+                torch::Tensor i_bias, torch::Tensor f_bias, double cap,
+                torch::Tensor mem, torch::Tensor mstate,
+                torch::Tensor state_slots, torch::Tensor qlocs,
+                torch::Tensor seq_lens) {
+  CHECK_GPU(proj); CHECK_GPU(o); CHECK_F32(o); CHECK_CONTIG(o);
+  CHECK_GPU(em); CHECK_F32(em); CHECK_CONTIG(em);
+  CHECK_GPU(mem); CHECK_F32(mem); CHECK_CONTIG(mem);
+  CHECK_GPU(mstate); CHECK_F32(mstate); CHECK_CONTIG(mstate);
+  CHECK_GPU(i_bias); CHECK_F32(i_bias); CHECK_GPU(f_bias); CHECK_F32(f_bias);
+  CHECK_I32(state_slots); CHECK_I32(qlocs); CHECK_I32(seq_lens);
+  TORCH_CHECK(mem.dim() == 4 && o.dim() == 3, "state and read-out ranks");
+  const long T = proj.size(0), H = mem.size(1), dk = mem.size(2);
+  const long dv = mem.size(3) - 1, S = seq_lens.numel();
+  TORCH_CHECK(dk <= 256 && dv >= 1, "key size above 256 is unsupported");
+  TORCH_CHECK(o.size(0) == T && o.size(1) == H && o.size(2) == dv + 1 &&
+              em.numel() == T * H && mstate.dim() == 2 &&
+              mstate.size(0) == mem.size(0) && mstate.size(1) == H &&
+              i_bias.numel() == H && f_bias.numel() == H &&
+              qlocs.numel() == S + 1 && state_slots.numel() == S,
+              "operand sizes");
+  check_proj(proj, q_off, H * dk, "q");
+  check_proj(proj, k_off, H * dk, "k");
+  check_proj(proj, v_off, H * dv, "v");
+  check_proj(proj, i_off, H, "input gate");
+  check_proj(proj, f_off, H, "forget gate");
+  auto scratch = torch::empty({2, T, H}, o.options());
+  float* fa = scratch.data_ptr<float>();
+  mix_mlstm_scan(o.data_ptr<float>(), em.data_ptr<float>(), fa, fa + T * H,
+                 proj.data_ptr(), proj.stride(0), (int)q_off, (int)k_off,
+                 (int)v_off, (int)i_off, (int)f_off, i_bias.data_ptr<float>(),
+                 f_bias.data_ptr<float>(), (float)cap, mem.data_ptr<float>(),
+                 mstate.data_ptr<float>(), state_slots.data_ptr<int>(),
+                 qlocs.data_ptr<int>(), seq_lens.data_ptr<int>(), (int)S,
+                 (int)H, (int)dk, (int)dv, act_kind(proj), cur_stream());
+}
+
+void mlstm_out(torch::Tensor out, long out_off, torch::Tensor o,
+               torch::Tensor em, torch::Tensor norm_w, torch::Tensor proj,
+               long g_off, double eps) {
+  CHECK_GPU(o); CHECK_F32(o); CHECK_CONTIG(o); CHECK_GPU(em); CHECK_F32(em);
+  CHECK_CONTIG(em); CHECK_GPU(norm_w); CHECK_F32(norm_w); CHECK_CONTIG(norm_w);
+  CHECK_GPU(out); CHECK_GPU(proj);
+  const long T = o.size(0), H = o.size(1), dv = o.size(2) - 1;
+  TORCH_CHECK(norm_w.numel() == H * dv && em.numel() == T * H,
+              "parameter sizes");
+  TORCH_CHECK(out.dim() == 2 && out.stride(1) == 1 && out.size(0) == T &&
+              out_off >= 0 && out_off + H * dv <= out.size(1), "out section");
+  TORCH_CHECK(out.scalar_type() == proj.scalar_type() && proj.size(0) == T,
+              "dtype or row mismatch");
+  check_proj(proj, g_off, H * dv, "gate");
+  mix_mlstm_out(out.data_ptr(), out.stride(0), (int)out_off,
+                o.data_ptr<float>(), em.data_ptr<float>(),
+                norm_w.data_ptr<float>(), proj.data_ptr(), proj.stride(0),
+                (int)g_off, (float)eps, T, (int)H, (int)dv, act_kind(out),
+                cur_stream());
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("gelu_tanh_mul", &gelu_tanh_mul, "tanh-GELU(gate) * up");
   m.def("gated_norm_residual", &gated_norm_residual,
@@ -340,7 +613,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("chunk"), py::arg("window"), py::arg("proj"),
         py::arg("gate_off"), py::arg("out_scale"),
         py::arg("tile_seq") = c10::nullopt, py::arg("tile_q0") = c10::nullopt,
-        py::arg("prefill_rows") = 0);
+        py::arg("prefill_rows") = 0, py::arg("bias_r1") = c10::nullopt,
+        py::arg("bias_r2") = c10::nullopt);
   m.def("delta_prep", &delta_prep, "delta-rule inputs: filters, norms, gates",
         py::arg("qn"), py::arg("kn"), py::arg("v"), py::arg("decay"),
         py::arg("beta"), py::arg("proj"), py::arg("q_off"), py::arg("k_off"),
@@ -351,4 +625,17 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("conv_wt") = c10::nullopt);
   m.def("delta_scan", &delta_scan, "gated delta rule over new tokens");
   m.def("delta_out", &delta_out, "per-head norm + low-rank gate of the read-out");
+  m.def("token_embed", &token_embed,
+        "token row + hashed-bigram row + position sinusoid, fp32");
+  m.def("weighted_rmsnorm", &weighted_rmsnorm, "RMS norm with a weight vector");
+  m.def("norm_residual", &norm_residual,
+        "post-norm + residual (+ depth-weighted sum) (+ next pre-norm)");
+  m.def("poly_act", &poly_act, "PolyNorm activation");
+  m.def("tied_attn_prep", &tied_attn_prep,
+        "whole-projection q/k norm, query temperature, K and raw-K page write");
+  m.def("section_rmsnorm", &section_rmsnorm,
+        "RMS norm of a projection section, optionally scattered by row index");
+  m.def("sigmoid_gate_mul", &sigmoid_gate_mul, "v *= sigmoid(gate section)");
+  m.def("mlstm_scan", &mlstm_scan, "mLSTM memory over new tokens");
+  m.def("mlstm_out", &mlstm_out, "mLSTM read-out normalisation, norm and gate");
 }

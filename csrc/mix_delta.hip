@@ -278,27 +278,6 @@ __global__ void conv_state_update_kernel(
 
 #define TB 8    // tokens staged per step
 
-// sum over the R adjacent lanes of a column (R = 1, 2, 4, 8 or 16, aligned):
-// DPP moves inside the VALU, no LDS round trip. quad_perm covers the xor-1
-// and xor-2 steps; after them every lane of a quad holds the quad's sum, so
-// the mirror steps (lane i <- lane 7-i, then 15-i) complete rows of 8 and 16.
-template <int R>
-__device__ __forceinline__ float group_sum(float v) {
-  if (R >= 2)
-    v += __int_as_float(__builtin_amdgcn_update_dpp(
-        0, __float_as_int(v), 0xB1, 0xF, 0xF, true));   // quad_perm 1,0,3,2
-  if (R >= 4)
-    v += __int_as_float(__builtin_amdgcn_update_dpp(
-        0, __float_as_int(v), 0x4E, 0xF, 0xF, true));   // quad_perm 2,3,0,1
-  if (R >= 8)
-    v += __int_as_float(__builtin_amdgcn_update_dpp(
-        0, __float_as_int(v), 0x141, 0xF, 0xF, true));  // row_half_mirror
-  if (R >= 16)
-    v += __int_as_float(__builtin_amdgcn_update_dpp(
-        0, __float_as_int(v), 0x140, 0xF, 0xF, true));  // row_mirror
-  return v;
-}
-
 // Token-by-token scan. Block = (sequence, head, group of 256/R columns);
 // lane (col, r) keeps rows {((n/4)*R + r)*4 + n%4 : n < RPT} of its column of
 // S in registers (RPT = 32, or 16 to double the number of waves when a

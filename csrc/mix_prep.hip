@@ -1,0 +1,139 @@
+// Projection post-processing of attention variants that norm a whole
+// projection at once:
+//   tied_attn_prep    q and k sections RMS-normed over ALL heads together
+//                     (weights of the section's size); q times a temperature
+//                     1 + coef * ln(floor((p + 1) / every) + 1) of its
+//                     position p; normed k into the paged K cache and the RAW
+//                     k section into the paged V cache (values are the keys)
+//   section_rmsnorm   out[row(t)] = n(section of proj[t]) * w; row(t) = t, or
+//                     an index list (scatter into cache pages: a latent)
+//   sigmoid_gate_mul  v *= sigmoid(gate section), elementwise
+// One 256-thread block a token (and section); fp32 math.
+#include "mix_common.h"
+
+template <typename A>
+__global__ void tied_attn_prep_kernel(
+    A* __restrict__ q_out, const A* __restrict__ proj, long ld, int q_off,
+    int k_off, const float* __restrict__ q_w, const float* __restrict__ k_w,
+    float eps, const long* __restrict__ pos, float temp_coef, int temp_every,
+    const long* __restrict__ slots, A* __restrict__ k_cache,
+    A* __restrict__ v_cache, int H, int G, int dk, int page) {
+  __shared__ float red[4];
+  const long t = blockIdx.x;
+  const bool is_q = blockIdx.y == 0;
+  const int n = (is_q ? H : G) * dk;
+  const A* src = proj + t * ld + (is_q ? q_off : k_off);
+  float ssq = 0.f;
+  for (int c = threadIdx.x; c < n; c += blockDim.x) {
+    const float v = ldf<A>(src + c);
+    ssq += v * v;
+  }
+  float inv = 1.f / sqrtf(block_sum_256(ssq, red) / (float)n + eps);
+  if (is_q) {
+    if (temp_every > 0) {
+      const long steps = (pos[t] + 1) / temp_every;
+      inv *= 1.f + temp_coef * logf((float)steps + 1.f);
+    }
+    A* dst = q_out + t * (long)n;
+    for (int c = threadIdx.x; c < n; c += blockDim.x)
+      stf<A>(dst + c, ldf<A>(src + c) * q_w[c] * inv);
+    return;
+  }
+  const long slot = slots[t];
+  const long blk = slot / page, off = slot - blk * page;
+  for (int c = threadIdx.x; c < n; c += blockDim.x) {
+    const int g = c / dk, i = c - g * dk;
+    const long at = ((blk * G + g) * page + off) * (long)dk + i;
+    const float v = ldf<A>(src + c);
+    stf<A>(k_cache + at, v * inv * k_w[c]);
+    stf<A>(v_cache + at, v);
+  }
+}
+
+template <typename A>
+__global__ void section_rmsnorm_kernel(A* __restrict__ out, long ldo,
+                                       const A* __restrict__ proj, long ld,
+                                       int off, const float* __restrict__ w,
+                                       float eps, const long* __restrict__ rows,
+                                       int n) {
+  __shared__ float red[4];
+  const long t = blockIdx.x;
+  const A* src = proj + t * ld + off;
+  float ssq = 0.f;
+  for (int c = threadIdx.x; c < n; c += blockDim.x) {
+    const float v = ldf<A>(src + c);
+    ssq += v * v;
+  }
+  const float inv = 1.f / sqrtf(block_sum_256(ssq, red) / (float)n + eps);
+  A* dst = out + (rows ? rows[t] : t) * ldo;
+  for (int c = threadIdx.x; c < n; c += blockDim.x)
+    stf<A>(dst + c, ldf<A>(src + c) * inv * w[c]);
+}
+
+template <typename A>
+__global__ void sigmoid_gate_mul_kernel(A* __restrict__ v, long ldv,
+                                        const A* __restrict__ proj, long ld,
+                                        int g_off, long T, int N) {
+  const long total = T * (long)N;
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (long)gridDim.x * blockDim.x) {
+    const long row = idx / N;
+    const int c = (int)(idx - row * N);
+    A* p = v + row * ldv + c;
+    stf<A>(p, ldf<A>(p) * sigmoid_f(ldf<A>(proj + row * ld + g_off + c)));
+  }
+}
+
+extern "C" void mix_tied_attn_prep(void* q_out, const void* proj, long ld,
+                                   int q_off, int k_off, const float* q_w,
+                                   const float* k_w, float eps,
+                                   const long* pos, float temp_coef,
+                                   int temp_every, const long* slots,
+                                   void* k_cache, void* v_cache, long T, int H,
+                                   int G, int dk, int page, int f32,
+                                   hipStream_t s) {
+  if (T == 0) return;
+  const dim3 grid((unsigned)T, 2);
+  if (f32)
+    hipLaunchKernelGGL(tied_attn_prep_kernel<float>, grid, dim3(256), 0, s,
+                       (float*)q_out, (const float*)proj, ld, q_off, k_off,
+                       q_w, k_w, eps, pos, temp_coef, temp_every, slots,
+                       (float*)k_cache, (float*)v_cache, H, G, dk, page);
+  else
+    hipLaunchKernelGGL(tied_attn_prep_kernel<u16>, grid, dim3(256), 0, s,
+                       (u16*)q_out, (const u16*)proj, ld, q_off, k_off, q_w,
+                       k_w, eps, pos, temp_coef, temp_every, slots,
+                       (u16*)k_cache, (u16*)v_cache, H, G, dk, page);
+}
+
+extern "C" void mix_section_rmsnorm(void* out, long ldo, const void* proj,
+                                    long ld, int off, const float* w,
+                                    float eps, const long* rows, long T, int n,
+                                    int f32, hipStream_t s) {
+  if (T == 0) return;
+  if (f32)
+    hipLaunchKernelGGL(section_rmsnorm_kernel<float>, dim3((unsigned)T),
+                       dim3(256), 0, s, (float*)out, ldo, (const float*)proj,
+                       ld, off, w, eps, rows, n);
+  else
+    hipLaunchKernelGGL(section_rmsnorm_kernel<u16>, dim3((unsigned)T),
+                       dim3(256), 0, s, (u16*)out, ldo, (const u16*)proj, ld,
+                       off, w, eps, rows, n);
+}
+
+extern "C" void mix_sigmoid_gate_mul(void* v, long ldv, const void* proj,
+                                     long ld, int g_off, long T, int N,
+                                     int f32, hipStream_t s) {
+  const long total = T * (long)N;
+  if (total == 0) return;
+  long blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  if (f32)
+    hipLaunchKernelGGL(sigmoid_gate_mul_kernel<float>, dim3((unsigned)blocks),
+                       dim3(256), 0, s, (float*)v, ldv, (const float*)proj, ld,
+                       g_off, T, N);
+  else
+    hipLaunchKernelGGL(sigmoid_gate_mul_kernel<u16>, dim3((unsigned)blocks),
+                       dim3(256), 0, s, (u16*)v, ldv, (const u16*)proj, ld,
+                       g_off, T, N);
+}

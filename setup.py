@@ -34,6 +34,9 @@ MIX_SOURCES = [
     "csrc/mix_attn.hip",
     "csrc/mix_attn_mfma.hip",
     "csrc/mix_delta.hip",
+    "csrc/mix_stream.hip",
+    "csrc/mix_prep.hip",
+    "csrc/mix_mlstm.hip",
 ]
 
 # hipcc's automatic packed-fp32 forms are switched off for all device code

@@ -476,9 +476,9 @@ def tied_attn_prep(proj, q_off, k_off, H, G, dk, q_w, k_w, eps, positions,
     q = _unit_rms(q, eps) * q_w.float()
     kn = _unit_rms(k.float(), eps) * k_w.float()
     if temp_every > 0:
-        p = positions.to(torch.float32)
+        steps = torch.div(positions + 1, temp_every, rounding_mode="floor")
         q = q * (1.0 + temp_coef * torch.log(
-            torch.floor((p + 1.0) / float(temp_every)) + 1.0)).unsqueeze(1)
+            steps.to(torch.float32) + 1.0)).unsqueeze(1)
     bs = k_cache.shape[2]
     blk = slot_mapping // bs
     off = slot_mapping % bs

@@ -386,6 +386,8 @@ def test_window_edges_stand_out(backend, layout, mode, page):
         qn = (O.unit_rms(q.reshape(T, -1).double(), eps) * qw).view(T, H, dk)
         qn = qn * O.query_temperature(T, 0.25, 4)[:, None, None]
         kn = (O.unit_rms(k.reshape(T, -1).double(), eps) * kw).view(T, G, dk)
+        if dtype != torch.float32:  # as the query rows and the K pages hold them
+            qn, kn = (t.to(dtype).double() for t in (qn, kn))
         want = torch.stack([
             O.softmax_attention(qn[:, h], kn[:, h // (H // G)],
                                 k[:, h // (H // G)].double(), scale, vis,

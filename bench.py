@@ -78,6 +78,9 @@ def build_args():
                         "the Qwen3 dense decoder of equal size, random "
                         "weights (comma list of 1b,8b,tiny); one JSON line "
                         "per model")
+    p.add_argument("--compare-models", type=str, default="vodinex,qwen3",
+                   help="models of --arch-compare: comma list of vodinex, "
+                        "ruludra, qwen3")
     p.add_argument("--compare-seqs", type=int, default=16)
     p.add_argument("--compare-prompt", type=int, default=2048)
     p.add_argument("--e2e-rows", type=int, default=3000,
@@ -254,7 +257,8 @@ def main():
 
         rows = run_compare(args.arch_compare.split(","), device,
                            args.compare_seqs, args.compare_prompt,
-                           steps=args.steps, warmup=args.warmup)
+                           steps=args.steps, warmup=args.warmup,
+                           models=args.compare_models.split(","))
         if rank == 0:
             for r in rows:
                 print(json.dumps(r))

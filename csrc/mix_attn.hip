@@ -16,7 +16,9 @@
 // Positions count from the start of the sequence, so a chunk edge does not
 // move when a prompt is processed in pieces.
 //
-// One wave per (token, head) for both kernels; all math fp32.
+// attn_prep and the general local_attention kernel use one wave per (token,
+// head); shapes made of 16-byte vectors take the row-split kernel further
+// down. All math fp32.
 #include "mix_common.h"
 
 #define WPB 4  // waves per block
@@ -290,6 +292,167 @@ __global__ void local_attention_kernel(
   }
 }
 
+
+// ---- row-split kernel ------------------------------------------------------
+// One 4-wave block per (token, head); the visible keys are cut into tiles that
+// the waves take in turn, and the four partial (max, sum, accumulator)
+// triples meet in LDS. Inside a wave, LPR adjacent lanes own one cached row
+// (16 bytes a lane: 8 bf16 or 4 fp32), so one load instruction fetches whole
+// rows of 64 / LPR keys, fully coalesced; the partial dot products are summed
+// over the LPR lanes by xor-shuffles, which leaves every lane of a row group
+// with its key's score, and the same lanes then weight their 16-byte chunk of
+// the value row. This is the kernel of single-token (decode) rows: with a
+// window of W keys a row costs W / (4 * 64 / LPR) dependent steps instead of
+// W. Needs dk and dv to be multiples of the 16-byte vector and at most
+// 64 vectors long; other shapes take the one-wave kernel above.
+template <typename A> struct Vec16;
+template <> struct Vec16<u16> { typedef u16x8 type; };
+template <> struct Vec16<float> { typedef f32x4 type; };
+
+template <typename A, int LPR>
+__global__ void __launch_bounds__(256) local_attention_rows_kernel(
+    A* __restrict__ out, long ldo, int out_off, const A* __restrict__ q,
+    const A* __restrict__ k_cache, const A* __restrict__ v_cache,
+    const int* __restrict__ bt, int bt_stride, const int* __restrict__ seq_lens,
+    const int* __restrict__ qlocs, const int* __restrict__ token_seq,
+    float scale, int chunk, int window, const A* __restrict__ proj, long ld,
+    int gate_off, float out_scale, const float* __restrict__ bias_r1,
+    const float* __restrict__ bias_r2, long t0, int H, int G, int dk, int dv,
+    int page) {
+  typedef typename Vec16<A>::type vec_t;
+  constexpr int EPL = 16 / sizeof(A);     // elements per lane
+  constexpr int KPI = 64 / LPR;           // keys per load instruction
+  constexpr int TS = LPR < 16 ? LPR : 16; // steps per tile
+  constexpr int TK = TS * KPI;            // keys per tile
+  constexpr int DP = LPR * EPL;           // padded row length
+  constexpr int CS = 2 + DP;              // floats a wave leaves in LDS
+  __shared__ float qs[DP];
+  __shared__ float comb[WPB * CS];
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int wid = threadIdx.x / WAVE;
+  const int kg = lane / LPR, c0 = (lane % LPR) * EPL;
+  const long u = blockIdx.x;
+  const long t = t0 + u / H;
+  const int h = (int)(u % H);
+  const int g = h / (H / G);
+  for (int i = threadIdx.x; i < DP; i += blockDim.x)
+    qs[i] = i < dk ? ldf<A>(q + (t * H + h) * (long)dk + i) : 0.f;
+  __syncthreads();
+  float qr[EPL];
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) qr[e] = qs[c0 + e];
+
+  const int s = token_seq[t];
+  const int p = seq_lens[s] - (qlocs[s + 1] - (int)t);  // position of token t
+  int lo = 0;
+  if (chunk > 0) lo = (p / chunk) * chunk;
+  if (window > 0 && p - window + 1 > lo) lo = p - window + 1;
+  const int* table = bt + (long)s * bt_stride;
+  const float r1 = bias_r1 ? bias_r1[h] : 0.f;
+  const float r2 = bias_r1 ? bias_r2[h] : 0.f;
+  const bool kact = c0 < dk, vact = c0 < dv;
+
+  float m = -INFINITY, l = 0.f;
+  float acc[EPL];
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) acc[e] = 0.f;
+
+  const int n_tiles = (p - lo) / TK + 1;
+  for (int tile = wid; tile < n_tiles; tile += WPB) {
+    const int base = lo + tile * TK;
+    float sc[TS];
+    long vrow[TS];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int st = 0; st < TS; ++st) {
+      const int j = base + st * KPI + kg;
+      const bool live = j <= p;
+      float dot = 0.f;
+      long cell = 0;  // (blk * G + g) * page + off
+      if (live) {
+        const int blk = table[j / page];
+        cell = ((long)blk * G + g) * page + j % page;
+        if (kact) {
+          const vec_t kx = *(const vec_t*)(k_cache + cell * dk + c0);
+#pragma unroll
+          for (int e = 0; e < EPL; ++e) {
+            A ke = kx[e];
+            dot += qr[e] * ldf<A>(&ke);
+          }
+        }
+      }
+#pragma unroll
+      for (int o = LPR / 2; o > 0; o >>= 1) dot += __shfl_xor(dot, o, WAVE);
+      float sv = -INFINITY;
+      if (live) {
+        sv = dot * scale;
+        if (bias_r1) sv -= r1 * logf(1.f + r2 * (float)(p - j));
+      }
+      sc[st] = sv;
+      vrow[st] = cell;
+      tmax = fmaxf(tmax, sv);
+    }
+#pragma unroll
+    for (int o = LPR; o < 64; o <<= 1)
+      tmax = fmaxf(tmax, __shfl_xor(tmax, o, WAVE));
+    const float m_new = fmaxf(m, tmax);   // finite: key `base` is visible
+    const float corr = expf(m - m_new);   // m = -inf on the first tile -> 0
+    l *= corr;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) acc[e] *= corr;
+    m = m_new;
+#pragma unroll
+    for (int st = 0; st < TS; ++st) {
+      if (sc[st] == -INFINITY) continue;
+      const float pj = expf(sc[st] - m_new);
+      l += pj;
+      if (vact) {
+        const vec_t vx = *(const vec_t*)(v_cache + vrow[st] * dv + c0);
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+          A ve = vx[e];
+          acc[e] += pj * ldf<A>(&ve);
+        }
+      }
+    }
+  }
+  // key groups of the wave
+#pragma unroll
+  for (int o = LPR; o < 64; o <<= 1) {
+    l += __shfl_xor(l, o, WAVE);
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) acc[e] += __shfl_xor(acc[e], o, WAVE);
+  }
+  float* mine = comb + wid * CS;
+  if (lane < LPR) {
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) mine[2 + c0 + e] = acc[e];
+    if (lane == 0) {
+      mine[0] = m;
+      mine[1] = l;
+    }
+  }
+  __syncthreads();
+  float mx = comb[0];  // wave 0 always has a tile
+#pragma unroll
+  for (int w = 1; w < WPB; ++w) mx = fmaxf(mx, comb[w * CS]);
+  float wgt[WPB], lsum = 0.f;
+#pragma unroll
+  for (int w = 0; w < WPB; ++w) {
+    wgt[w] = expf(comb[w * CS] - mx);   // a wave without tiles: exp(-inf) = 0
+    lsum += wgt[w] * comb[w * CS + 1];
+  }
+  float gate = out_scale;
+  if (gate_off >= 0) gate *= sigmoid_f(ldf<A>(proj + t * ld + gate_off + h));
+  const float f = gate / lsum;
+  for (int c = threadIdx.x; c < dv; c += blockDim.x) {
+    float o = 0.f;
+#pragma unroll
+    for (int w = 0; w < WPB; ++w) o += wgt[w] * comb[w * CS + 2 + c];
+    stf<A>(out + t * ldo + out_off + (long)h * dv + c, o * f);
+  }
+}
+
 extern "C" void mix_attn_prep(void* q_out, const void* proj, long ld,
                               int q_off, int k_off, int v_off,
                               const float* q_w, const float* k_w, float eps,
@@ -344,6 +507,30 @@ static void launch_local_attention(
   const long units = T * H;
   const int grid = (int)((units + WPB - 1) / WPB);
   if (grid == 0) return;
+  {
+    constexpr int EPL = 16 / (int)sizeof(A);
+    const int dmax = dk > dv ? dk : dv;
+    if (dk % EPL == 0 && dv % EPL == 0 && dmax <= 64 * EPL) {
+      int lpr = 2;
+      while (lpr * EPL < dmax) lpr <<= 1;
+#define LAUNCH_LR(LL)                                                         \
+  hipLaunchKernelGGL((local_attention_rows_kernel<A, LL>),                    \
+                     dim3((unsigned)units), dim3(WPB * WAVE), 0, s, (A*)out,  \
+                     ldo, out_off, (const A*)q, (const A*)k_cache,            \
+                     (const A*)v_cache, bt, bt_stride, seq_lens, qlocs,       \
+                     token_seq, scale, chunk, window, (const A*)proj, ld,     \
+                     gate_off, out_scale, bias_r1, bias_r2, t0, H, G, dk, dv, \
+                     page)
+      if (lpr == 2) LAUNCH_LR(2);
+      else if (lpr == 4) LAUNCH_LR(4);
+      else if (lpr == 8) LAUNCH_LR(8);
+      else if (lpr == 16) LAUNCH_LR(16);
+      else if (lpr == 32) LAUNCH_LR(32);
+      else LAUNCH_LR(64);
+#undef LAUNCH_LR
+      return;
+    }
+  }
   const size_t smem = (size_t)WPB * dk * sizeof(float);
 #define LAUNCH_LA(NV)                                                        \
   hipLaunchKernelGGL((local_attention_kernel<A, NV>), dim3(grid),            \

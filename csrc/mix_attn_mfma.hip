@@ -49,12 +49,13 @@ __global__ void local_attention_mfma_kernel(
     const int* __restrict__ tile_q0, float scale, int chunk, int window,
     const u16* __restrict__ proj, long ld, int gate_off, float out_scale,
     const float* __restrict__ bias_r1, const float* __restrict__ bias_r2, int H,
-    int Hk, int dk, int dv) {
+    int Hk, int dk, int dv, int parts) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int w = threadIdx.x / WAVE;
-  const int G = blockDim.x / WAVE;
-  const int kh = blockIdx.y;
-  const int hq = kh * G + w;
+  const int G = blockDim.x / WAVE;        // query heads of this workgroup
+  // the query heads of one kv head are spread over `parts` workgroups
+  const int kh = blockIdx.y / parts;
+  const int hq = (kh * parts + blockIdx.y % parts) * G + w;
   const int s = tile_seq[blockIdx.x];
   const int q0 = tile_q0[blockIdx.x];
   const int row_base = qlocs[s] + q0;
@@ -223,22 +224,30 @@ extern "C" int mix_local_attention_mfma(
     int H, int Hk, int dk, int dv, int page, hipStream_t s) {
   if (page != PG || dk % 8 || dv % 8 || dk > 256 || dv > 256 || H % Hk)
     return 0;
-  const int G = H / Hk;
-  if (G > 16) return 0;
   const int DKP = dk <= 64 ? 64 : (dk <= 128 ? 128 : 256);
   const int DVP = dv <= 64 ? 64 : (dv <= 128 ? 128 : 256);
-  const size_t smem = (size_t)PG * DKP * 2 + (size_t)DVP * VPAD * 2 +
-                      (size_t)G * QT * VPAD * 2 + (size_t)G * 2 * QT * 4;
-  if (smem > 64 * 1024) return 0;
+  // one wave a query head; many query heads on one kv head (one shared
+  // latent, say) are split over several workgroups so that the tiles fit LDS
+  int G = H / Hk, parts = 1;
+  size_t smem = 0;
+  for (;; ++parts) {
+    if (parts > H / Hk) return 0;
+    if ((H / Hk) % parts) continue;
+    G = H / Hk / parts;
+    smem = (size_t)PG * DKP * 2 + (size_t)DVP * VPAD * 2 +
+           (size_t)G * QT * VPAD * 2 + (size_t)G * 2 * QT * 4;
+    if (G <= 8 && smem <= 64 * 1024) break;
+  }
   if (n_tiles == 0) return 1;
 #define LAUNCH_M(KP, VP)                                                      \
   hipLaunchKernelGGL((local_attention_mfma_kernel<KP, VP>),                   \
-                     dim3(n_tiles, Hk), dim3(G * WAVE), smem, s, (u16*)out,   \
+                     dim3(n_tiles, Hk * parts), dim3(G * WAVE), smem, s,      \
+                     (u16*)out,                                               \
                      ldo, out_off, (const u16*)q, (const u16*)k_cache,        \
                      (const u16*)v_cache, bt, bt_stride, seq_lens, qlocs,     \
                      tile_seq, tile_q0, scale, chunk, window,                 \
                      (const u16*)proj, ld, gate_off, out_scale, bias_r1,     \
-                     bias_r2, H, Hk, dk, dv)
+                     bias_r2, H, Hk, dk, dv, parts)
   if (DKP == 64) {
     if (DVP == 64) LAUNCH_M(64, 64);
     else if (DVP == 128) LAUNCH_M(64, 128);

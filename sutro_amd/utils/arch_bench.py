@@ -1,5 +1,5 @@
-"""Prefill and decode throughput of a layer-list decoder beside the Qwen3
-dense decoder of equal size (same width, layers, heads, key/value heads, head
+"""Prefill and decode throughput of the layer-list decoders (Vodinex,
+Ruludra) beside the Qwen3 dense decoder of equal size (same width, layers, heads, key/value heads, head
 size and feed-forward width), both with random weights, both through the
 engine's own batch path (scheduler, paged cache, state slots, decode
 hipGraphs). Used by `bench.py --arch-compare`.
@@ -20,7 +20,8 @@ from ..engine.config import EngineConfig
 from ..engine.engine import LLMEngine
 from ..models.hybrid_spec import (AttnMixerSpec, DeltaMixerSpec,
                                   HybridLayerSpec, HybridSpec,
-                                  ParallelMixerSpec)
+                                  LatentAttnMixerSpec, MLSTMMixerSpec,
+                                  ParallelMixerSpec, TiedAttnMixerSpec)
 from ..models.registry import ModelSpec
 
 # name -> (width, layers, heads, kv_heads, head size, ff, vocab)
@@ -49,6 +50,43 @@ def hybrid_spec(name: str, chunk: int = 1024) -> HybridSpec:
     return HybridSpec(name=f"vodinex-{name}", arch="vodinex", hidden_size=W,
                       vocab_size=V, layers=tuple(layers), norm_eps=1e-6,
                       residual_mult=0.8, max_context=1 << 20)
+
+
+def sandwich_spec(name: str, window: int = 1024) -> HybridSpec:
+    """Ruludra at the same width, depth, heads, head size and feed-forward
+    width: tied-value window attention, latent attention (latent 256, query
+    latent W/2), an mLSTM layer without feed-forward, and a latent layer that
+    reads the first one's cached latent, in turn."""
+    W, L, H, G, D, ff, V = SIZES[name]
+    rank = min(256, 2 * D)
+    attn = TiedAttnMixerSpec(heads=H, kv_heads=G, dim=D, scale=D ** -0.5,
+                             window=window, temp_coef=0.3, temp_every=64)
+    lat = LatentAttnMixerSpec(heads=H, dim=D, vdim=D, q_rank=W // 2,
+                              kv_rank=rank, scale=D ** -0.5, window=window)
+    rec = MLSTMMixerSpec(heads=max(1, H // 2), dim=D, vdim=D, gate_cap=15.0)
+    layers: List[HybridLayerSpec] = []
+    for i in range(L):
+        k = i % 4
+        if k == 0:
+            layers.append(HybridLayerSpec("attention", attn, ff=ff,
+                                          ff_kind="poly_norm"))
+        elif k == 1:
+            layers.append(HybridLayerSpec("latent_attention", lat, ff=ff,
+                                          ff_kind="poly_norm"))
+        elif k == 2:
+            layers.append(HybridLayerSpec("mlstm", rec, ff=0,
+                                          ff_kind="poly_norm"))
+        else:
+            layers.append(HybridLayerSpec(
+                "latent_attention",
+                LatentAttnMixerSpec(heads=H, dim=D, vdim=D, q_rank=W // 2,
+                                    kv_rank=rank, scale=D ** -0.5,
+                                    window=window, kv_from=i - 2),
+                ff=ff, ff_kind="poly_norm"))
+    return HybridSpec(name=f"ruludra-{name}", arch="ruludra", hidden_size=W,
+                      vocab_size=V, layers=tuple(layers), norm_eps=1e-6,
+                      max_context=1 << 20, bigram=(65521, 31, 17),
+                      pos_base=10000.0, logit_scale=0.25)
 
 
 def dense_spec(name: str) -> ModelSpec:
@@ -109,12 +147,17 @@ def _measure(spec, device: str, seqs: int, prompt: int, steps: int,
     return out
 
 
+MAKERS = {"vodinex": hybrid_spec, "qwen3": dense_spec,
+          "ruludra": sandwich_spec}
+
+
 def run_compare(sizes: List[str], device: str, seqs: int, prompt: int,
-                steps: int, warmup: int) -> List[dict]:
+                steps: int, warmup: int,
+                models=("vodinex", "qwen3")) -> List[dict]:
     rows = []
     for name in sizes:
-        for kind, spec in (("vodinex", hybrid_spec(name)),
-                           ("qwen3", dense_spec(name))):
+        for kind in models:
+            spec = MAKERS[kind](name)
             r = _measure(spec, device, seqs, prompt, steps, warmup)
             r.update(model=spec.name, kind=kind, size=name, seqs=seqs,
                      prompt=prompt, params=spec.param_count())

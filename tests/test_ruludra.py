@@ -343,7 +343,7 @@ def test_far_memory_survives_portions_and_decoding(tmp_path_factory, backend):
     check(ck, got, seqs, backend[1])
 
 
-@pytest.mark.parametrize("layout", ["tied", "latent"])
+@pytest.mark.parametrize("layout", ["tied", "latent", "latent_wide"])
 @pytest.mark.parametrize("mode", ["prompt", "decoded"])
 @pytest.mark.parametrize("page", [4, 8, 32])
 def test_window_edges_stand_out(backend, layout, mode, page):
@@ -352,15 +352,18 @@ def test_window_edges_stand_out(backend, layout, mode, page):
     token's window, at and next to page borders, or far back. The output must
     be that key's value when it is visible and must not contain it when it is
     not. `tied`: whole-projection norms, values = raw keys, distance bias.
-    `latent`: one shared latent read as key and value by every head."""
+    `latent`: one shared latent read as key and value by every head
+    (`latent_wide`: sixteen heads on a latent of 256)."""
     device, dtype = backend
     window = 11
     T = 75
     g = torch.Generator().manual_seed(11)
     if layout == "tied":
         H, G, dk = 4, 2, 8
-    else:
+    elif layout == "latent":
         H, G, dk = 3, 1, 16
+    else:       # many heads on one wide latent
+        H, G, dk = 16, 1, 256
     k = torch.randn(T, G, dk, generator=g) * 0.1
     q = torch.randn(T, H, dk, generator=g) * 0.1
     probes = []

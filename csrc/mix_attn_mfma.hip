@@ -40,8 +40,12 @@ __device__ __forceinline__ int kswz(int row, int byte_in_row) {
   return row * (2 * DKP) + (byte_in_row ^ ((row & mask & 15) << 4));
 }
 
+// Wide tiles (DKP + DVP > 256) keep 128 accumulator and 64 query registers a
+// lane: they run with at most 4 waves a workgroup so that a wave may use the
+// whole register file of its SIMD.
 template <int DKP, int DVP>
-__global__ void local_attention_mfma_kernel(
+__global__ void __launch_bounds__(DKP + DVP > 256 ? 256 : 1024)
+local_attention_mfma_kernel(
     u16* __restrict__ out, long ldo, int out_off, const u16* __restrict__ q,
     const u16* __restrict__ k_cache, const u16* __restrict__ v_cache,
     const int* __restrict__ bt, int bt_stride, const int* __restrict__ seq_lens,
@@ -236,7 +240,7 @@ extern "C" int mix_local_attention_mfma(
     G = H / Hk / parts;
     smem = (size_t)PG * DKP * 2 + (size_t)DVP * VPAD * 2 +
            (size_t)G * QT * VPAD * 2 + (size_t)G * 2 * QT * 4;
-    if (G <= 8 && smem <= 64 * 1024) break;
+    if (G <= (DKP + DVP > 256 ? 4 : 8) && smem <= 64 * 1024) break;
   }
   if (n_tiles == 0) return 1;
 #define LAUNCH_M(KP, VP)                                                      \

@@ -17,8 +17,8 @@
 // mlstm_scan maps the state onto lanes by COLUMN, like the delta-rule scan: a
 // column of C is owned by R adjacent lanes holding dk/R rows each in
 // registers; one token costs one R-lane sum (DPP moves) and broadcast reads
-// of the staged k and q rows. Blocks cover (sequence, head, group of
-// columns). A sequence whose first token (position 0) is in the batch starts
+// of the staged k and q rows. Blocks cover (sequence, head, group of value
+// columns); a fifth wave of the first group's block carries the normaliser. A sequence whose first token (position 0) is in the batch starts
 // from zero, whatever its slot held. Everything is fp32 except the
 // projection sections, which arrive in the activation type.
 #include "mix_common.h"
@@ -79,14 +79,14 @@ __global__ void mlstm_gates_kernel(
 }
 
 template <typename A, int R, int RPT>
-__global__ void __launch_bounds__(256) mlstm_scan_kernel(
+__global__ void __launch_bounds__(320) mlstm_scan_kernel(
     float* __restrict__ o, const A* __restrict__ proj, long ld, int q_off,
     int k_off, int v_off, const float* __restrict__ fa,
     const float* __restrict__ ib, float* __restrict__ mem,
     const int* __restrict__ state_slots, const int* __restrict__ qlocs,
     const int* __restrict__ seq_lens, int H, int dk, int dv, int col_groups) {
   constexpr int DKP = R * RPT;
-  constexpr int CPB = 256 / R;             // columns per block
+  constexpr int CPB = 256 / R;             // value columns per block
   constexpr int NK = 2 * MTB * DKP / 256;  // staged k|q floats per lane
   constexpr int NV = MTB * CPB / 256 > 0 ? MTB * CPB / 256 : 1;
   constexpr int TILE = 2 * MTB * DKP + MTB * CPB + MTB;
@@ -97,11 +97,17 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(
   const int h = b % H;
   const int s = b / H;
   const int tid = threadIdx.x;
+  // Waves 0-3 own the value columns of this group and stage the tiles. Wave
+  // 4 exists for the normaliser (column dv of the state, whose "value" is
+  // 1): its first R lanes own it in the first column group; everywhere else
+  // the wave only keeps the barriers company. The value columns thus fill
+  // whole groups (dv = 128 -> 4 groups, not 5 with one lane row in use).
+  const bool extra = tid >= 256;
   const int r = tid % R;
-  const int cl = tid / R;                  // column within the block
-  const int col = cg * CPB + cl;
-  const int dv1 = dv + 1;                  // column dv is the normaliser
-  const bool cv = col < dv1;
+  const int cl = (tid & 255) / R;          // column within the block
+  const int dv1 = dv + 1;
+  const int col = extra ? dv : cg * CPB + cl;
+  const bool cv = extra ? (cg == 0 && tid - 256 < R) : col < dv;
   const int q0 = qlocs[s], q1 = qlocs[s + 1];
   if (q1 <= q0) return;
   const int start = seq_lens[s] - (q1 - q0);
@@ -117,6 +123,7 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(
 
   float pk[NK], pv[NV], pf = 0.f;
   auto prefetch = [&](int t0) {
+    if (extra) return;
 #pragma unroll
     for (int n = 0; n < NK; ++n) {
       const int e = tid + n * 256;
@@ -138,10 +145,8 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(
       const int e = tid + n * 256;
       const int tok = e / CPB, c = cg * CPB + e % CPB;
       const int t = t0 + tok;
-      float x = 0.f;
-      if (e < MTB * CPB && t < q1 && c < dv1)
-        x = c < dv ? ldf<A>(proj + (long)t * ld + v_off + h * dv + c) : 1.f;
-      pv[n] = x;
+      pv[n] = (e < MTB * CPB && t < q1 && c < dv)
+                  ? ldf<A>(proj + (long)t * ld + v_off + h * dv + c) : 0.f;
     }
     if (tid < MTB) pf = t0 + tid < q1 ? fa[(long)(t0 + tid) * H + h] : 1.f;
   };
@@ -150,19 +155,22 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(
   int buf = 0;
   for (int t0 = q0; t0 < q1; t0 += MTB, buf ^= 1) {
     float* L = lds[buf];
+    if (!extra) {
 #pragma unroll
-    for (int n = 0; n < NK; ++n) L[tid + n * 256] = pk[n];
+      for (int n = 0; n < NK; ++n) L[tid + n * 256] = pk[n];
 #pragma unroll
-    for (int n = 0; n < NV; ++n)
-      if (tid + n * 256 < MTB * CPB) L[2 * MTB * DKP + tid + n * 256] = pv[n];
-    if (tid < MTB) L[2 * MTB * DKP + MTB * CPB + tid] = pf;
+      for (int n = 0; n < NV; ++n)
+        if (tid + n * 256 < MTB * CPB) L[2 * MTB * DKP + tid + n * 256] = pv[n];
+      if (tid < MTB) L[2 * MTB * DKP + MTB * CPB + tid] = pf;
+    }
     __syncthreads();
     if (t0 + MTB < q1) prefetch(t0 + MTB);
+    if (!cv) continue;                     // wave-uniform except in wave 4
     const int nt = min(MTB, q1 - t0);
     for (int tok = 0; tok < nt; ++tok) {
       const f32x4* K4 = (const f32x4*)(L + tok * DKP);
       const f32x4* Q4 = (const f32x4*)(L + (MTB + tok) * DKP);
-      const float vt = L[2 * MTB * DKP + tok * CPB + cl];
+      const float vt = extra ? 1.f : L[2 * MTB * DKP + tok * CPB + cl];
       const float ft = L[2 * MTB * DKP + MTB * CPB + tok];
       float out = 0.f;
 #pragma unroll
@@ -175,7 +183,7 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(
         }
       }
       out = group_sum<R>(out);
-      if (r == 0 && cv) o[((long)(t0 + tok) * H + h) * dv1 + col] = out;
+      if (r == 0) o[((long)(t0 + tok) * H + h) * dv1 + col] = out;
     }
   }
   if (cv) {
@@ -243,7 +251,7 @@ extern "C" void mix_mlstm_scan(float* o, float* em, float* fa, float* ib,
   int rpt = 32;
   {
     // few sequences x heads: 16 rows a lane doubles the waves in flight
-    const long blocks32 = (long)S * H * ((dv + 1 + 256 / R - 1) / (256 / R));
+    const long blocks32 = (long)S * H * ((dv + 256 / R - 1) / (256 / R));
     if (blocks32 < 512 && dk > 16) {
       rpt = 16;
       R = 2;
@@ -251,11 +259,11 @@ extern "C" void mix_mlstm_scan(float* o, float* em, float* fa, float* ib,
     }
   }
   const int cols_pb = 256 / R;
-  const int col_groups = (dv + 1 + cols_pb - 1) / cols_pb;
+  const int col_groups = (dv + cols_pb - 1) / cols_pb;
   const long grid = (long)S * H * col_groups;
 #define LAUNCH_MS(AA, RR, PP)                                                 \
   hipLaunchKernelGGL((mlstm_scan_kernel<AA, RR, PP>), dim3((unsigned)grid),   \
-                     dim3(256), 0, s, o, (const AA*)proj, ld, q_off, k_off,   \
+                     dim3(320), 0, s, o, (const AA*)proj, ld, q_off, k_off,   \
                      v_off, fa, ib, mem, state_slots, qlocs, seq_lens, H, dk, \
                      dv, col_groups)
 #define PICK_MS(AA)                                                      \

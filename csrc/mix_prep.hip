@@ -84,6 +84,33 @@ __global__ void sigmoid_gate_mul_kernel(A* __restrict__ v, long ldv,
   }
 }
 
+// 16-byte form: needs N, both row strides and the gate offset to be multiples
+// of the vector (8 bf16 or 4 fp32)
+template <typename A, int V>
+__global__ void sigmoid_gate_mul_vec_kernel(A* __restrict__ v, long ldv,
+                                            const A* __restrict__ proj,
+                                            long ld, int g_off, long T, int N) {
+  typedef A vec_t __attribute__((ext_vector_type(V)));
+  const int vpr = N / V;
+  const long total = T * (long)vpr;
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (long)gridDim.x * blockDim.x) {
+    const long row = idx / vpr;
+    const int c = (int)(idx - row * vpr) * V;
+    vec_t* p = (vec_t*)(v + row * ldv + c);
+    const vec_t x = *p;
+    const vec_t g = *(const vec_t*)(proj + row * ld + g_off + c);
+    vec_t o;
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      A xj = x[j], gj = g[j], r;
+      stf<A>(&r, ldf<A>(&xj) * sigmoid_f(ldf<A>(&gj)));
+      o[j] = r;
+    }
+    *p = o;
+  }
+}
+
 extern "C" void mix_tied_attn_prep(void* q_out, const void* proj, long ld,
                                    int q_off, int k_off, const float* q_w,
                                    const float* k_w, float eps,
@@ -126,6 +153,21 @@ extern "C" void mix_sigmoid_gate_mul(void* v, long ldv, const void* proj,
                                      int f32, hipStream_t s) {
   const long total = T * (long)N;
   if (total == 0) return;
+  const int V = f32 ? 4 : 8;
+  if (N % V == 0 && ldv % V == 0 && ld % V == 0 && g_off % V == 0 &&
+      (size_t)v % 16 == 0 && (size_t)proj % 16 == 0) {
+    long vb = (total / V + 255) / 256;
+    if (vb > 65536) vb = 65536;
+    if (f32)
+      hipLaunchKernelGGL((sigmoid_gate_mul_vec_kernel<float, 4>),
+                         dim3((unsigned)vb), dim3(256), 0, s, (float*)v, ldv,
+                         (const float*)proj, ld, g_off, T, N);
+    else
+      hipLaunchKernelGGL((sigmoid_gate_mul_vec_kernel<u16, 8>),
+                         dim3((unsigned)vb), dim3(256), 0, s, (u16*)v, ldv,
+                         (const u16*)proj, ld, g_off, T, N);
+    return;
+  }
   long blocks = (total + 255) / 256;
   if (blocks > 65536) blocks = 65536;
   if (f32)

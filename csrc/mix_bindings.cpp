@@ -389,7 +389,7 @@ void token_embed(torch::Tensor out, torch::Tensor ids,
   const float* fp = nullptr;
   if (inv_freq.has_value()) {
     CHECK_GPU(*inv_freq); CHECK_F32(*inv_freq); CHECK_CONTIG(*inv_freq);
-    TORCH_CHECK(W % 2 == 0 && inv_freq->numel() == W / 2, "sinusoid table");
+    TORCH_CHECK(inv_freq->numel() == (W + 1) / 2, "sinusoid table");
     fp = inv_freq->data_ptr<float>();
   }
   mix_token_embed(out.data_ptr<float>(), ids.data_ptr<long>(), pp,

@@ -143,8 +143,6 @@ class RuludraModel(nn.Module):
         if spec.bigram:
             self.bigram = nn.Embedding(spec.bigram[0] + 1, W, dtype=dtype)
         if spec.pos_base:
-            if W % 2:
-                raise ValueError("the sinusoid needs an even width")
             self.register_buffer(
                 "pos_inv_freq", hops.sinusoid_inv_freq(W, spec.pos_base),
                 persistent=False)

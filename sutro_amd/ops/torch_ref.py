@@ -401,8 +401,8 @@ def delta_out(o, norm_w, proj, g1_off, g2, eps, out, out_off, out_scale):
 
 
 def sinusoid_inv_freq(width: int, base: float) -> torch.Tensor:
-    """fp32 [width/2]: base^(-2i/width), rounded once from fp64."""
-    i = torch.arange(width // 2, dtype=torch.float64)
+    """fp32 [ceil(width/2)]: base^(-2i/width), rounded once from fp64."""
+    i = torch.arange((width + 1) // 2, dtype=torch.float64)
     return (float(base) ** (-2.0 * i / width)).float()
 
 
@@ -419,7 +419,8 @@ def token_embed(ids, prev_ids, positions, embed_w, bigram_w, buckets: int,
         x = x + bigram_w[row].float()
     if inv_freq is not None:
         ang = positions.to(torch.float32).unsqueeze(1) * inv_freq.unsqueeze(0)
-        x = x + torch.stack([ang.sin(), ang.cos()], dim=-1).reshape(x.shape[0], -1)
+        x = x + torch.stack([ang.sin(), ang.cos()],
+                            dim=-1).reshape(x.shape[0], -1)[:, :x.shape[1]]
     return x
 
 

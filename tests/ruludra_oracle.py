@@ -37,11 +37,11 @@ def bigram_rows(tokens, buckets, mul_prev, mul_cur):
 def sinusoid(T, width):
     """[T, width]: column 2i = sin(p / 10000^(2i/width)), column 2i+1 = cos."""
     p = torch.arange(T, dtype=F64)[:, None]
-    i = torch.arange(width // 2, dtype=F64)[None, :]
+    i = torch.arange((width + 1) // 2, dtype=F64)[None, :]
     ang = p * 10000.0 ** (-2.0 * i / width)
     out = torch.zeros(T, width, dtype=F64)
     out[:, 0::2] = torch.sin(ang)
-    out[:, 1::2] = torch.cos(ang)
+    out[:, 1::2] = torch.cos(ang)[:, :width // 2]
     return out
 
 

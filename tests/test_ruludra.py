@@ -343,6 +343,36 @@ def test_far_memory_survives_portions_and_decoding(tmp_path_factory, backend):
     check(ck, got, seqs, backend[1])
 
 
+@pytest.mark.parametrize("n,off", [(12, 3), (64, 8), (1032, 16)])
+def test_section_norm_scatter_and_gate(backend, n, off):
+    """Norm of a projection section into rows chosen by an index list (a
+    latent into its pages) and the elementwise sigmoid gate, for sizes that
+    take the plain and the 16-byte forms."""
+    device, dtype = backend
+    T = 9
+    g = torch.Generator().manual_seed(n)
+    proj = torch.randn(T, off + 2 * n + 8, generator=g).to(dtype)
+    w = torch.rand(n, generator=g) + 0.5
+    rows = torch.tensor([5, 0, 19, 7, 2, 11, 3, 18, 9])
+    want = O.unit_rms(proj[:, off:off + n].double(), 1e-5) * w
+    pages = torch.full((20, n), 3.0, dtype=dtype, device=device)
+    hops.section_rmsnorm(proj.to(device), off, n, w.to(device), 1e-5, pages,
+                         rows=rows.to(device))
+    tol = 1e-5 if dtype == torch.float32 else 3e-2
+    assert float((pages[rows].double().cpu() - want).abs().max()) < tol
+    untouched = [i for i in range(20) if i not in rows.tolist()]
+    assert float((pages[untouched].float() - 3.0).abs().max()) == 0.0
+    dense = torch.empty(T, n, dtype=dtype, device=device)
+    hops.section_rmsnorm(proj.to(device), off, n, w.to(device), 1e-5, dense)
+    assert float((dense.double().cpu() - want).abs().max()) < tol
+    buf = torch.randn(T, n + 8, generator=g).to(dtype)
+    v = buf.clone().to(device)
+    hops.sigmoid_gate_mul(v[:, :n], proj.to(device), off + n)
+    gate = torch.sigmoid(proj[:, off + n:off + 2 * n].double())
+    assert float((v[:, :n].double().cpu() - buf[:, :n].double() * gate).abs().max()) < tol
+    assert float((v[:, n:].float().cpu() - buf[:, n:].float()).abs().max()) == 0.0
+
+
 @pytest.mark.parametrize("layout", ["tied", "latent", "latent_wide"])
 @pytest.mark.parametrize("mode", ["prompt", "decoded"])
 @pytest.mark.parametrize("page", [4, 8, 32])
@@ -456,12 +486,13 @@ def test_window_edges_stand_out(backend, layout, mode, page):
         assert float((want[i, h] - vals[j, h // (H // G)].double()).abs().max()) > 0.5
 
 
-def test_bigram_rows_and_positions(backend):
+@pytest.mark.parametrize("W", [24, 15])
+def test_bigram_rows_and_positions(backend, W):
     """The embedding alone: hashed rows with collisions, the extra row for a
     first token, previous tokens handed over between pieces, positions far
-    from zero."""
+    from zero, an odd width (the last column has a sine and no cosine)."""
     device, dtype = backend
-    W, V, buckets = 24, 40, 7
+    V, buckets = 40, 7
     g = torch.Generator().manual_seed(4)
     emb = torch.randn(V, W, generator=g).to(dtype)
     big = torch.randn(buckets + 1, W, generator=g).to(dtype)
@@ -534,11 +565,14 @@ def test_mlstm_stabiliser_and_denominator(backend):
     assert float(mem[1].min()) == 7.0          # other slots untouched
 
 
-def test_sandwich_norms_depth_sum_and_polynorm(backend):
+@pytest.mark.parametrize("W,F", [(40, 52), (38, 64), (2056, 4104)])
+def test_sandwich_norms_depth_sum_and_polynorm(backend, W, F):
     """The fused post-norm + residual + depth-weighted sum + pre-norm, and
-    PolyNorm, against their equations."""
+    PolyNorm, against their equations; row lengths that take the plain
+    kernels and the register-resident vector forms with one and more chunks
+    a thread."""
     device, dtype = backend
-    T, W, F, n = 7, 40, 52, 4
+    T, n = 7, 4
     g = torch.Generator().manual_seed(8)
     X = torch.randn(n, T, W, generator=g) * 3
     x_in = torch.randn(T, W, generator=g) * 3
@@ -555,7 +589,7 @@ def test_sandwich_norms_depth_sum_and_polynorm(backend):
     hops.norm_residual(xw, y.to(device), wb.to(device), eps, Xd[n - 1],
                        stack=Xd, depth_w=dw.to(device), mix_out=xw,
                        next_w=wn.to(device), h_out=h)
-    tol = 1e-5 if dtype == torch.float32 else 3e-2
+    tol = 2e-5 if dtype == torch.float32 else 3e-2
     assert float((Xd[n - 1].double().cpu() - r).abs().max()) < 1e-5
     assert float((xw.double().cpu() - z).abs().max()) < 1e-5
     assert float((h.double().cpu() - h_want).abs().max()) < tol
@@ -602,6 +636,16 @@ def test_greedy_generation_through_scheduler(tmp_path_factory, backend):
             assert tok == best or margin < 20 * limit(dtype), (n, tok, best)
             checked += 1
     assert checked >= 20
+
+
+def test_service_job_on_a_checkpoint_directory(tmp_path_factory, local_client):
+    """A checkpoint directory is a model name for the job service too."""
+    ck = checkpoint(tmp_path_factory, "config_a", config_a)
+    job = local_client.infer(["alpha", "beta gamma"], model=ck[0],
+                             sampling_params={"max_tokens": 4, "temperature": 0},
+                             stay_attached=False)
+    out = local_client.await_job_completion(job, timeout=120)
+    assert out is not None and len(out) == 2
 
 
 def test_cli_generates_from_a_checkpoint_directory(tmp_path_factory):

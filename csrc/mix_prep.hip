@@ -70,6 +70,42 @@ __global__ void section_rmsnorm_kernel(A* __restrict__ out, long ldo,
     stf<A>(dst + c, ldf<A>(src + c) * inv * w[c]);
 }
 
+// 16-byte form: one vector a thread (sections up to 256 vectors long), the
+// section is read once. Needs n, the offset and both row strides to be
+// multiples of the vector (8 bf16 or 4 fp32).
+template <typename A, int V>
+__global__ void __launch_bounds__(256) section_rmsnorm_vec_kernel(
+    A* __restrict__ out, long ldo, const A* __restrict__ proj, long ld,
+    int off, const float* __restrict__ w, float eps,
+    const long* __restrict__ rows, int n) {
+  typedef A vec_t __attribute__((ext_vector_type(V)));
+  __shared__ float red[4];
+  const long t = blockIdx.x;
+  const int c = threadIdx.x * V;
+  float x[V];
+  float ssq = 0.f;
+  if (c < n) {
+    const vec_t v = *(const vec_t*)(proj + t * ld + off + c);
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      A ve = v[e];
+      x[e] = ldf<A>(&ve);
+      ssq += x[e] * x[e];
+    }
+  }
+  const float inv = 1.f / sqrtf(block_sum_256(ssq, red) / (float)n + eps);
+  if (c < n) {
+    vec_t o;
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      A oe;
+      stf<A>(&oe, x[e] * inv * w[c + e]);
+      o[e] = oe;
+    }
+    *(vec_t*)(out + (rows ? rows[t] : t) * ldo + c) = o;
+  }
+}
+
 template <typename A>
 __global__ void sigmoid_gate_mul_kernel(A* __restrict__ v, long ldv,
                                         const A* __restrict__ proj, long ld,
@@ -138,6 +174,19 @@ extern "C" void mix_section_rmsnorm(void* out, long ldo, const void* proj,
                                     float eps, const long* rows, long T, int n,
                                     int f32, hipStream_t s) {
   if (T == 0) return;
+  const int V = f32 ? 4 : 8;
+  if (n % V == 0 && n <= 256 * V && off % V == 0 && ld % V == 0 &&
+      ldo % V == 0 && (size_t)out % 16 == 0 && (size_t)proj % 16 == 0) {
+    if (f32)
+      hipLaunchKernelGGL((section_rmsnorm_vec_kernel<float, 4>),
+                         dim3((unsigned)T), dim3(256), 0, s, (float*)out, ldo,
+                         (const float*)proj, ld, off, w, eps, rows, n);
+    else
+      hipLaunchKernelGGL((section_rmsnorm_vec_kernel<u16, 8>),
+                         dim3((unsigned)T), dim3(256), 0, s, (u16*)out, ldo,
+                         (const u16*)proj, ld, off, w, eps, rows, n);
+    return;
+  }
   if (f32)
     hipLaunchKernelGGL(section_rmsnorm_kernel<float>, dim3((unsigned)T),
                        dim3(256), 0, s, (float*)out, ldo, (const float*)proj,

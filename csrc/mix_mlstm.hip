@@ -121,7 +121,12 @@ __global__ void __launch_bounds__(320) mlstm_scan_kernel(
     C[n] = (start > 0 && cv && i < dk) ? Cg[(long)i * dv1 + col] : 0.f;
   }
 
-  float pk[NK], pv[NV], pf = 0.f;
+  // The prefetch only LOADS: raw elements and raw scale factors stay in
+  // registers untouched until they are written to LDS one tile later, so no
+  // wait for memory stands between the loads and the arithmetic of the
+  // current tile.
+  A rk[NK], rv[NV];
+  float rs[NK], pf = 0.f;
   auto prefetch = [&](int t0) {
     if (extra) return;
 #pragma unroll
@@ -130,23 +135,26 @@ __global__ void __launch_bounds__(320) mlstm_scan_kernel(
       const int arr = e / (MTB * DKP), rem = e % (MTB * DKP);
       const int tok = rem / DKP, i = rem % DKP;
       const int t = t0 + tok;
-      float x = 0.f;
+      A x = (A)0;            // all-zero bits are 0.0 in both element types
+      float sc = qscale;
       if (t < q1 && i < dk) {
-        if (arr == 0)
-          x = ldf<A>(proj + (long)t * ld + k_off + h * dk + i) *
-              ib[(long)t * H + h];
-        else
-          x = ldf<A>(proj + (long)t * ld + q_off + h * dk + i) * qscale;
+        if (arr == 0) {
+          x = proj[(long)t * ld + k_off + h * dk + i];
+          sc = ib[(long)t * H + h];
+        } else {
+          x = proj[(long)t * ld + q_off + h * dk + i];
+        }
       }
-      pk[n] = x;
+      rk[n] = x;
+      rs[n] = sc;
     }
 #pragma unroll
     for (int n = 0; n < NV; ++n) {
       const int e = tid + n * 256;
       const int tok = e / CPB, c = cg * CPB + e % CPB;
       const int t = t0 + tok;
-      pv[n] = (e < MTB * CPB && t < q1 && c < dv)
-                  ? ldf<A>(proj + (long)t * ld + v_off + h * dv + c) : 0.f;
+      rv[n] = (e < MTB * CPB && t < q1 && c < dv)
+                  ? proj[(long)t * ld + v_off + h * dv + c] : (A)0;
     }
     if (tid < MTB) pf = t0 + tid < q1 ? fa[(long)(t0 + tid) * H + h] : 1.f;
   };
@@ -157,17 +165,21 @@ __global__ void __launch_bounds__(320) mlstm_scan_kernel(
     float* L = lds[buf];
     if (!extra) {
 #pragma unroll
-      for (int n = 0; n < NK; ++n) L[tid + n * 256] = pk[n];
+      for (int n = 0; n < NK; ++n)
+        L[tid + n * 256] = ldf<A>(&rk[n]) * rs[n];
 #pragma unroll
       for (int n = 0; n < NV; ++n)
-        if (tid + n * 256 < MTB * CPB) L[2 * MTB * DKP + tid + n * 256] = pv[n];
+        if (tid + n * 256 < MTB * CPB)
+          L[2 * MTB * DKP + tid + n * 256] = ldf<A>(&rv[n]);
       if (tid < MTB) L[2 * MTB * DKP + MTB * CPB + tid] = pf;
     }
     __syncthreads();
     if (t0 + MTB < q1) prefetch(t0 + MTB);
     if (!cv) continue;                     // wave-uniform except in wave 4
     const int nt = min(MTB, q1 - t0);
-    for (int tok = 0; tok < nt; ++tok) {
+#pragma unroll
+    for (int tok = 0; tok < MTB; ++tok) {
+      if (tok >= nt) break;
       const f32x4* K4 = (const f32x4*)(L + tok * DKP);
       const f32x4* Q4 = (const f32x4*)(L + (MTB + tok) * DKP);
       const float vt = extra ? 1.f : L[2 * MTB * DKP + tok * CPB + cl];

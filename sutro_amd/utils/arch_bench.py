@@ -60,10 +60,10 @@ def sandwich_spec(name: str, window: int = 1024) -> HybridSpec:
     W, L, H, G, D, ff, V = SIZES[name]
     rank = min(256, 2 * D)
     attn = TiedAttnMixerSpec(heads=H, kv_heads=G, dim=D, scale=D ** -0.5,
-                             window=window, temp_coef=0.3, temp_every=64)
+                             window=window, temp_coef=0.2, temp_every=128)
     lat = LatentAttnMixerSpec(heads=H, dim=D, vdim=D, q_rank=W // 2,
                               kv_rank=rank, scale=D ** -0.5, window=window)
-    rec = MLSTMMixerSpec(heads=max(1, H // 2), dim=D, vdim=D, gate_cap=15.0)
+    rec = MLSTMMixerSpec(heads=max(1, H // 2), dim=D, vdim=D, gate_cap=10.0)
     layers: List[HybridLayerSpec] = []
     for i in range(L):
         k = i % 4
@@ -85,8 +85,8 @@ def sandwich_spec(name: str, window: int = 1024) -> HybridSpec:
                 ff=ff, ff_kind="poly_norm"))
     return HybridSpec(name=f"ruludra-{name}", arch="ruludra", hidden_size=W,
                       vocab_size=V, layers=tuple(layers), norm_eps=1e-6,
-                      max_context=1 << 20, bigram=(65521, 31, 17),
-                      pos_base=10000.0, logit_scale=0.25)
+                      max_context=1 << 20, bigram=(65521, 131, 7),
+                      pos_base=10000.0, logit_scale=0.5)
 
 
 def dense_spec(name: str) -> ModelSpec:

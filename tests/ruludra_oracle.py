@@ -205,7 +205,7 @@ def forward(config, w, tokens, streams=None):
 
 # -------------------------------------------------- configs and weights -----
 
-def attn_cfg(heads, kv_heads, dim, window, scale, coef=0.3, every=16):
+def attn_cfg(heads, kv_heads, dim, window, scale, coef=0.25, every=16):
     return {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim,
             "mask": {"size": window}, "scale": scale,
             "q_temp": {"coef": coef, "every": every}}

@@ -85,12 +85,12 @@ def config_c():
     latent sizes that are multiples of 8), windows longer than a page and
     not a multiple of it."""
     return O.make_config(64, 300, [
-        O.layer("attention", O.attn_cfg(4, 2, 32, 40, 0.18, coef=0.3, every=16), ff=96),
+        O.layer("attention", O.attn_cfg(4, 2, 32, 40, 0.18, coef=0.35, every=16), ff=96),
         O.layer("latent_attention", O.latent_cfg(4, 16, 24, 32, 32, 33, 0.25), ff=64),
         O.layer("mlstm", O.mlstm_cfg(2, 32, 40, cap=10.0)),
         O.layer("latent_attention", O.latent_cfg(2, 32, 16, 16, 32, 70, 0.2, kv_from=1)),
         O.layer("attention", O.attn_cfg(2, 2, 64, 35, 0.12, coef=0.2, every=7), ff=48),
-    ], eps=1e-6, logit_scale=0.3, buckets=509, mul_prev=31, mul_cur=3)
+    ], eps=1e-6, logit_scale=0.3, buckets=509, mul_prev=29, mul_cur=3)
 
 
 _CACHE = {}
@@ -256,6 +256,72 @@ def test_long_decoding(tmp_path_factory, backend):
     seqs = {"s": tokens_for(ck[1], 124, 3)}
     got = replay(eng, seqs, [[("s", 4)]] + [[("s", 1)]] * 120)
     check(ck, got, seqs, backend[1])
+
+
+# ------------------------------------------------ random configurations -----
+
+def random_config(seed):
+    """Widths, head counts, head and latent sizes, windows, temperature
+    steps, gate caps, hash constants, the order of layers and which of them
+    have a feed-forward or borrow a latent: all drawn at random."""
+    import random
+
+    rnd = random.Random(seed)
+    layers, owners = [], []
+    for i in range(rnd.randint(3, 7)):
+        kind = rnd.choice(["attention", "latent_attention", "mlstm"])
+        ff = rnd.choice([None, 40, 72, 136])
+        win = rnd.choice([3, 16, 33, 50, 64])
+        if kind == "attention":
+            G = rnd.choice([1, 2, 4])
+            dim = rnd.choice([16, 24, 32, 40, 20])
+            m = O.attn_cfg(G * rnd.choice([1, 2, 3]), G, dim, win,
+                           dim ** -0.5 * rnd.choice([1.0, 0.7]),
+                           coef=rnd.choice([0.0, 0.2, 0.5]),
+                           every=rnd.choice([1, 7, 32]))
+        elif kind == "latent_attention":
+            dim = rnd.choice([16, 32, 24])
+            kr = rnd.choice([16, 32, 40, 72])
+            cands = [j for j in owners if layers[j]["mixer"]["kv_rank"] == kr]
+            src = rnd.choice(cands) if cands and rnd.random() < 0.6 else None
+            m = O.latent_cfg(rnd.choice([1, 2, 3, 6, 12]), dim,
+                             rnd.choice([16, 48, 36]), rnd.choice([24, 40, 64]),
+                             kr, win, dim ** -0.5, kv_from=src)
+            if src is None:
+                owners.append(i)
+        else:
+            m = O.mlstm_cfg(rnd.choice([1, 2, 5]), rnd.choice([16, 48, 24]),
+                            rnd.choice([16, 64, 40]),
+                            cap=rnd.choice([5.0, 12.0, 30.0]))
+        layers.append(O.layer(kind, m, ff=ff))
+    return O.make_config(rnd.choice([64, 96, 136]), rnd.choice([300, 512, 777]),
+                         layers, eps=rnd.choice([1e-6, 1e-5]),
+                         logit_scale=rnd.choice([0.2, 1.0, 2.0]),
+                         buckets=rnd.choice([97, 613, 4093]),
+                         mul_prev=rnd.choice([37, 7, 101]),
+                         mul_cur=rnd.choice([19, 3, 29]))
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3, 4])
+def test_random_configurations(tmp_path_factory, backend, seed):
+    """A drawn configuration through a mixed schedule (portions beside single
+    tokens, pages of 32, a pool smaller than the sum of the requests)."""
+    ck = checkpoint(tmp_path_factory, f"random{seed}",
+                    lambda: random_config(seed), seed=seed)
+    eng = engine(ck, backend, page=32, blocks=8, max_seqs=3)
+    seqs = {"a": tokens_for(ck[1], 90, seed), "b": tokens_for(ck[1], 31, seed + 1),
+            "c": tokens_for(ck[1], 47, seed + 2)}
+    schedule = [[("a", 40), ("b", 3)], [("a", 1), ("b", 20), ("c", 2)],
+                [("a", 30), ("b", 1), ("c", 1)], [("a", 2), ("b", 1), ("c", 40)],
+                [("a", 1), ("b", 1), ("c", 1)], [("a", 1), ("b", 1), ("c", 1)],
+                [("a", 15), ("b", 4), ("c", 2)]]
+    got = replay(eng, seqs, schedule)
+    for k in seqs:
+        rows = row_errors(got[k], oracle_logits(ck, seqs[k]))
+        if backend[1] == torch.float32:
+            assert float(rows.max()) < limit(backend[1]), (k, float(rows.max()))
+        else:   # single positions of a drawn model can be ill-conditioned
+            assert float(rows.mean()) < 3e-2, (k, float(rows.mean()))
 
 
 # ----------------------------------------------------- batches, reuse -------

@@ -2,7 +2,8 @@
 mixer and feed-forward, so attention layers, recurrent layers and layers that
 run both side by side can be ordered freely.
 
-A spec is built from a checkpoint's ``config.json`` (see :func:`vodinex_spec`)
+A spec is built from a checkpoint's ``config.json`` (see :func:`vodinex_spec`
+and :func:`ruludra_spec`)
 or directly in code (tests, benchmarks). Nothing here fixes a size: widths,
 head counts, mask sizes, filter lengths and the order of layers all come from
 the config.

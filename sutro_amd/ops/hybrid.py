@@ -1,6 +1,9 @@
 """Ops of layer-list ("hybrid") decoders: scalar-gain norms with gated
 residuals, tanh-GELU gating, local (chunked / windowed) paged attention with
-split key/value sizes and partial rotation, and the gated delta rule.
+split key/value sizes, partial rotation and an optional distance bias, the
+gated delta rule; hashed-bigram + sinusoid embedding, weighted norms around a
+sublayer with depth-weighted sums of all layer results, PolyNorm, tied-value
+attention prep, latent norms and gates, and the mLSTM.
 
 GPU tensors run the HIP kernels of the `sutro_amd._C_mix` extension
 (csrc/mix_*.hip), templated on the activation type: bf16 when the engine

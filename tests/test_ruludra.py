@@ -704,6 +704,26 @@ def test_greedy_generation_through_scheduler(tmp_path_factory, backend):
     assert checked >= 20
 
 
+def test_lagged_decode_generates_the_same_tokens(tmp_path_factory, backend):
+    """One-step-lagged decoding feeds the sampled-token tensor straight into
+    the next step; the token before it (for the bigram row) is then the
+    host's last known token. Greedy outputs must equal the synchronous ones."""
+    ck = checkpoint(tmp_path_factory, "config_a", config_a)
+    prompts = [tokens_for(ck[1], n, 50 + n) for n in (9, 4, 17)]
+    outs = []
+    for lagged in (False, True):
+        eng = engine(ck, backend, blocks=40, async_decode=lagged)
+        reqs = [eng.add_request(p, SamplingParams(max_tokens=10, temperature=0.0))
+                for p in prompts]
+        steps = 0
+        while eng.has_work():
+            eng.step()
+            steps += 1
+            assert steps < 200
+        outs.append([r.output_token_ids for r in reqs])
+    assert outs[0] == outs[1]
+
+
 def test_service_job_on_a_checkpoint_directory(tmp_path_factory, local_client):
     """A checkpoint directory is a model name for the job service too."""
     ck = checkpoint(tmp_path_factory, "config_a", config_a)
